@@ -285,6 +285,113 @@ class MoESpec:
         )
 
 
+@dataclass
+class LatentAttentionSpec:
+    """Attention whose keys and values are expanded per head from one cached
+    latent vector per token: the cache holds ``kv_rank`` normed latent
+    coordinates and (with ``rot_dim`` > 0) one rotated key part shared by all
+    heads. Queries go through a normed latent of ``q_rank`` coordinates and
+    have ``dim`` unrotated + ``rot_dim`` rotated coordinates per head.
+    ``window`` > 0: a query sees itself and the window-1 positions before it;
+    ``sink``: one more term exp(sink_h) in the softmax denominator; ``gate``:
+    head outputs times sigmoid of a projection of the sublayer input;
+    ``kv_from``: the layer has no latent projection and reads the cache of
+    that earlier layer."""
+
+    heads: int
+    dim: int
+    vdim: int
+    kv_rank: int
+    q_rank: int
+    scale: float
+    rot_dim: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    window: int = 0
+    sink: bool = False
+    gate: bool = False
+    kv_from: Optional[int] = None
+
+    @property
+    def cache_dim(self) -> int:
+        return self.kv_rank + self.rot_dim
+
+    @classmethod
+    def from_dict(cls, d: dict, sink: bool, gate: bool) -> "LatentAttentionSpec":
+        rot = d.get("rot") or {}
+        mask = d.get("mask") or {}
+        rot_dim = int(d.get("rot_dim", 0))
+        kv_from = d.get("kv_from")
+        return cls(
+            heads=int(d["heads"]),
+            dim=int(d["dim"]),
+            vdim=int(d.get("vdim", d["dim"])),
+            kv_rank=int(d["kv_rank"]),
+            q_rank=int(d["q_rank"]),
+            scale=float(d["scale"]),
+            rot_dim=rot_dim,
+            rot_dims=int(rot.get("dims", rot_dim)) if rot_dim else 0,
+            rot_base=float(rot.get("base", 10000.0)),
+            window=int(mask.get("size", 0)),
+            sink=sink,
+            gate=gate,
+            kv_from=None if kv_from is None else int(kv_from),
+        )
+
+
+@dataclass
+class MLPSpec:
+    """Plain two-matrix feed-forward with biases: down(act(up h + b) ) + b,
+    act = gelu in its tanh form."""
+
+    ff: int
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "MLPSpec":
+        return cls(ff=int(d["ff"]))
+
+
+@dataclass
+class SoftmaxMoESpec:
+    """Mixture of gated silu experts routed by softmax scores: the ``top``
+    experts by score + a per-expert correction are chosen, weighted by their
+    (uncorrected) scores renormalised to sum 1, and the weight multiplies the
+    expert's OUTPUT. The last ``identity`` router outputs stand for experts
+    that return their input; ``experts`` counts the real ones. An optional
+    shared expert of the same form runs for every token."""
+
+    experts: int
+    top: int
+    ff: int
+    identity: int = 0
+    shared_ff: int = 0
+
+    @property
+    def router_outputs(self) -> int:
+        return self.experts + self.identity
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "SoftmaxMoESpec":
+        r = d["router"]
+        sh = d.get("shared")
+        return cls(
+            experts=int(r["experts"]),
+            top=int(r["top"]),
+            ff=int(d["expert"]["ff"]),
+            identity=int(r.get("identity", 0)),
+            shared_ff=int(sh["ff"]) if sh else 0,
+        )
+
+
+def voborax_feed_forward_spec(d: Optional[dict]):
+    """``mlp`` entry of a Voborax layer -> MLPSpec, SoftmaxMoESpec or None."""
+    if not d:
+        return None
+    if d.get("kind", "moe" if "router" in d else "dense") == "moe":
+        return SoftmaxMoESpec.from_dict(d)
+    return MLPSpec.from_dict(d)
+
+
 def feed_forward_spec(d: Optional[dict]):
     """``mlp`` entry of a layer -> GLUSpec, MoESpec or None."""
     if not d:
@@ -313,9 +420,10 @@ class HybridLayerSpec:
     kind: str
     attention: Optional[AttentionMixerSpec] = None
     ssm: Optional[SSMMixerSpec] = None
+    latent: Optional[LatentAttentionSpec] = None
     attention_scale: float = 1.0
     ssm_scale: float = 1.0
-    mlp: Optional[object] = None  # GLUSpec or MoESpec
+    mlp: Optional[object] = None  # GLUSpec, MoESpec, MLPSpec or SoftmaxMoESpec
 
 
 @dataclass
@@ -335,6 +443,8 @@ class HybridModelConfig:
     num_local_experts: int = 0
     sliding_window: Optional[int] = None
     loop: Optional[LoopSpec] = None
+    # every sublayer output is multiplied by this before it joins the stream
+    residual_mult: float = 1.0
 
     @property
     def num_layers(self) -> int:
@@ -358,12 +468,15 @@ class HybridModelConfig:
         return any(l.ssm is not None for l in self.layers)
 
     def kv_bytes_per_block(self, block_size: int, itemsize: int) -> int:
-        return sum(
-            self.layers[i].attention.kv_heads
-            * (self.layers[i].attention.dim + self.layers[i].attention.vdim)
-            for i, _ in self.layer_runs()
-            if self.layers[i].attention is not None
-        ) * block_size * itemsize
+        per_token = 0
+        for i, _ in self.layer_runs():
+            a, lt = self.layers[i].attention, self.layers[i].latent
+            if a is not None:
+                per_token += a.kv_heads * (a.dim + a.vdim)
+            if lt is not None and lt.kv_from is None:
+                # one row per token: latent + shared rotated key part
+                per_token += lt.cache_dim
+        return per_token * block_size * itemsize
 
     @classmethod
     def from_dict(cls, cfg: dict, model_name: str = "merulorn") -> "HybridModelConfig":
@@ -371,6 +484,20 @@ class HybridModelConfig:
         for entry in cfg["layers"]:
             kind = entry["type"]
             mixer = entry["mixer"]
+            if kind in ("latent_attention", "latent_attention_2"):
+                # rotated key part + window + output gate, or none of them
+                # and a sink
+                first = kind == "latent_attention"
+                layers.append(
+                    HybridLayerSpec(
+                        kind,
+                        latent=LatentAttentionSpec.from_dict(
+                            mixer, sink=not first, gate=first
+                        ),
+                        mlp=voborax_feed_forward_spec(entry.get("mlp")),
+                    )
+                )
+                continue
             mlp = feed_forward_spec(entry.get("mlp"))
             if kind == "attention":
                 layers.append(
@@ -403,6 +530,7 @@ class HybridModelConfig:
             embedding_scale=float(cfg.get("embedding", {}).get("scale", 1.0)),
             model_name=model_name,
             architecture=cfg.get("architecture", "Merulorn"),
+            residual_mult=float(cfg.get("residual_mult", 1.0)),
             loop=(
                 LoopSpec(
                     start=int(cfg["loop"].get("start", 0)),

@@ -155,8 +155,10 @@ class ModelRunner:
             if kv is not None:
                 g, d, dv = kv
                 k = alloc((num_blocks, g, bs, d), dtype=dtype, device=self.device)
-                v = alloc((num_blocks, g, bs, dv), dtype=dtype, device=self.device)
-                kv_bytes += k.numel() * k.itemsize + v.numel() * v.itemsize
+                kv_bytes += k.numel() * k.itemsize
+                if dv:  # dv 0: the values are columns of the key rows
+                    v = alloc((num_blocks, g, bs, dv), dtype=dtype, device=self.device)
+                    kv_bytes += v.numel() * v.itemsize
             if state:
                 shape, dt = state["conv"]
                 conv = alloc((slots, *shape), dtype=dt, device=self.device)

@@ -24,7 +24,10 @@ from kserve_amd import ops
 from kserve_amd.engine.config import (
     AttentionMixerSpec,
     GLUSpec,
+    LatentAttentionSpec,
+    MLPSpec,
     MoESpec,
+    SoftmaxMoESpec,
     SSMMixerSpec,
 )
 from kserve_amd.ops.torch_ref import rotary_inv_freq
@@ -34,7 +37,8 @@ class LayerCache(NamedTuple):
     """What one layer keeps between steps; absent parts are None."""
 
     k: Optional[torch.Tensor] = None      # [blocks, kv_heads, block, dim]
-    v: Optional[torch.Tensor] = None      # [blocks, kv_heads, block, vdim]
+    v: Optional[torch.Tensor] = None      # [blocks, kv_heads, block, vdim];
+    #                                       None where values are read from k
     conv: Optional[torch.Tensor] = None   # [slots, taps-1, channels]
     ssm: Optional[torch.Tensor] = None    # [slots, heads, vdim, state] fp32
 
@@ -371,6 +375,263 @@ class RoutedClampedMoE(nn.Module):
         )
         idx, w, dense_w, _ = ops.route_tokens(
             h, self.router, self.spec.top, dense=dense
+        )
+        if dense:
+            return self._dense(h, dense_w, extra)
+        return self._sorted(h, idx, w, extra)
+
+
+class LatentAttention(nn.Module):
+    """Attention over one cached latent row per token. The sublayer input is
+    projected to [query latent | kv latent | key part | gate] in one GEMM;
+    both latents are RMS-normed, the key part is rotated in pairs (2i, 2i+1)
+    by the position, and [kv latent | rotated key part] is the only thing
+    written to the pages (one "kv head" of ``kv_rank + rot_dim`` columns).
+
+    Keys and values are never expanded. With k_h = U_k[h] c and v_h = U_v[h] c
+    the score q_h . k_h equals (U_k[h]^T q_h) . c, so every query head is
+    folded through its U_k[h] into latent coordinates (fp32) and attention
+    runs as multi-query attention against the cached rows, the latent part of
+    the row serving as the value; the weighted latent sum is then taken
+    through U_v[h] per head. Scores, weights, sink and the output gate
+    (a per-head scalar, so it commutes with U_v[h]) stay in the fp32
+    attention kernel.
+
+    Options: ``window`` (sliding), ``sink`` (softmax denominator term),
+    ``gate``, ``rot_dim`` = 0 (no positions at all), ``kv_from`` (no kv
+    projection: the layer attends to the pages of an earlier layer with its
+    own U_k / U_v)."""
+
+    # widest cached row the fp32 attention kernel takes
+    MAX_CACHE_DIM = 256
+
+    def __init__(self, width: int, spec: LatentAttentionSpec, eps: float, dtype):
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        self.dtype = dtype
+        s = spec
+        if s.rot_dims % 2 or s.rot_dims > s.rot_dim:
+            raise ValueError("rotated coordinates: even, at most the rotated part")
+        if s.cache_dim > self.MAX_CACHE_DIM:
+            raise NotImplementedError(
+                f"latent row of {s.cache_dim} columns (kv_rank + rot_dim): the "
+                f"attention kernel takes at most {self.MAX_CACHE_DIM}"
+            )
+        self.own_kv = s.kv_from is None
+        self.kv_cols = s.cache_dim if self.own_kv else 0
+        self.in_proj = _param(
+            s.q_rank + self.kv_cols + (s.heads if s.gate else 0), width, dtype=dtype
+        )
+        self.q_norm = _param(s.q_rank, dtype=torch.float32)
+        self.kv_norm = (
+            _param(s.kv_rank, dtype=torch.float32) if self.own_kv else None
+        )
+        self.uq = _param(s.heads * (s.dim + s.rot_dim), s.q_rank, dtype=dtype)
+        self.uk = _param(s.heads, s.dim, s.kv_rank, dtype=dtype)
+        # U_v stored transposed per head: [heads, kv_rank, vdim]
+        self.uv_t = _param(s.heads, s.kv_rank, s.vdim, dtype=dtype)
+        self.sink = _param(s.heads, dtype=torch.float32) if s.sink else None
+        self.o_proj = _param(width, s.heads * s.vdim, dtype=dtype)
+        self.register_buffer(
+            "inv_freq",
+            rotary_inv_freq(s.rot_dims, s.rot_base) if s.rot_dims else None,
+            persistent=False,
+        )
+
+    def load(self, get, prefix: str):
+        dt, s = self.dtype, self.spec
+        parts = [get(prefix + "dq").to(dt)]
+        if self.own_kv:
+            parts.append(get(prefix + "dkv").to(dt))
+            self.kv_norm.copy_(get(prefix + "dkv.norm").float())
+        if s.gate:
+            parts.append(get(prefix + "g").to(dt))
+        self.in_proj.copy_(torch.cat(parts, dim=0))
+        self.q_norm.copy_(get(prefix + "dq.norm").float())
+        self.uq.copy_(get(prefix + "uq").to(dt))
+        self.uk.copy_(get(prefix + "uk").to(dt).view(s.heads, s.dim, s.kv_rank))
+        self.uv_t.copy_(
+            get(prefix + "uv").to(dt).view(s.heads, s.vdim, s.kv_rank).transpose(1, 2)
+        )
+        if self.sink is not None:
+            self.sink.copy_(get(prefix + "sink").float())
+        self.o_proj.copy_(get(prefix + "o").to(dt))
+
+    def forward(self, h, positions, cache: LayerCache, meta):
+        """``cache.k``: this layer's pages, or those of layer ``kv_from``."""
+        s = self.spec
+        proj = F.linear(h, self.in_proj)
+        cq = ops.latent_norm_rope_cache(
+            proj, s.q_rank, s.kv_rank if self.own_kv else 0,
+            s.rot_dim if self.own_kv else 0, self.q_norm, self.kv_norm,
+            positions, meta.slot_mapping, cache.k if self.own_kv else None,
+            self.eps, self.inv_freq,
+        )
+        q = F.linear(cq, self.uq)
+        qf = ops.head_matmul_rope(
+            q, self.uk, s.heads, s.rot_dim, positions, self.inv_freq,
+            torch.float32,
+        )
+        gate = proj[:, s.q_rank + self.kv_cols :] if s.gate else None
+        o_lat = ops.ctx_attention_f32(
+            qf, cache.k, cache.k[..., : s.kv_rank], meta.block_tables,
+            meta.cu_seqlens, meta.context_lens, s.scale, meta.max_seqlen,
+            s.heads, gate=gate, out_dtype=self.dtype, sink=self.sink,
+            window=s.window,
+        )
+        o = ops.head_matmul_rope(o_lat, self.uv_t, s.heads)
+        return F.linear(o, self.o_proj)
+
+
+class GeluMLP(nn.Module):
+    """down(gelu_tanh(up h + b_up)) + b_down."""
+
+    def __init__(self, width: int, spec: MLPSpec, dtype):
+        super().__init__()
+        self.spec = spec
+        self.up = _param(spec.ff, width, dtype=dtype)
+        self.up_b = _param(spec.ff, dtype=torch.float32)
+        self.down = _param(width, spec.ff, dtype=dtype)
+        self.down_b = _param(width, dtype=dtype)
+
+    def load(self, get, prefix: str):
+        dt = self.up.dtype
+        self.up.copy_(get(prefix + "up").to(dt))
+        self.up_b.copy_(get(prefix + "up.b").float())
+        self.down.copy_(get(prefix + "down").to(dt))
+        self.down_b.copy_(get(prefix + "down.b").to(dt))
+
+    def forward(self, h):
+        a = ops.bias_gelu_tanh(F.linear(h, self.up), self.up_b)
+        return F.linear(a, self.down, self.down_b)
+
+
+class SiluGLU(nn.Module):
+    """down(silu(gate h) * (up h)), no biases; gate|up are one GEMM."""
+
+    def __init__(self, width: int, ff: int, dtype):
+        super().__init__()
+        self.gate_up = _param(2 * ff, width, dtype=dtype)
+        self.down = _param(width, ff, dtype=dtype)
+
+    def load(self, get, prefix: str):
+        dt = self.gate_up.dtype
+        self.gate_up.copy_(
+            torch.cat([get(prefix + "gate").to(dt), get(prefix + "up").to(dt)], dim=0)
+        )
+        self.down.copy_(get(prefix + "down").to(dt))
+
+    def forward(self, h):
+        return F.linear(ops.glu_silu_scale(F.linear(h, self.gate_up)), self.down)
+
+
+class SoftmaxRoutedMoE(nn.Module):
+    """Mixture of gated silu experts. fp32 router logits over
+    ``experts + identity`` outputs, softmax scores; the ``top`` outputs by
+    score + correction are chosen and weighted by their scores renormalised
+    to sum 1; the weight multiplies the expert's OUTPUT. An identity expert
+    returns the token's input. A shared expert is added for every token.
+
+    Weights: gate|up stacked as [E, 2 ff, width] (also one [E * 2 ff, width]
+    matrix), down as [width, E, ff] (also one [width, E * ff] matrix).
+    Small batches and captured decode graphs run every expert on every token:
+    ONE GEMM against all gate|up rows (the experts share their input), the
+    activation scaled by the token's weight for that expert (zero where it
+    was not chosen), ONE GEMM against all down columns, which also sums over
+    the experts in its fp32 accumulator. Larger batches sort the
+    (token, expert) pairs by expert and run a GEMM pair per expert on its
+    contiguous rows; the pairs of identity experts sort last and copy their
+    input rows."""
+
+    DENSE_ROW_BUDGET = RoutedClampedMoE.DENSE_ROW_BUDGET
+    RENORM_EPS = 1e-20
+
+    def __init__(self, width: int, spec: SoftmaxMoESpec, dtype):
+        super().__init__()
+        self.spec = spec
+        self.dtype = dtype
+        E, R = spec.experts, spec.router_outputs
+        if not 1 <= spec.top <= R:
+            raise ValueError("top must be between 1 and the router's outputs")
+        self.dense_max_tokens = max(16, self.DENSE_ROW_BUDGET * spec.top // max(E, 1))
+        self.router = _param(R, width, dtype=torch.float32)
+        self.correction = _param(R, dtype=torch.float32)
+        self.gate_up = _param(E, 2 * spec.ff, width, dtype=dtype)
+        self.down = _param(width, E, spec.ff, dtype=dtype)
+        self.shared = SiluGLU(width, spec.shared_ff, dtype) if spec.shared_ff else None
+
+    def load(self, get, prefix: str):
+        dt = self.dtype
+        self.router.copy_(get(prefix + "router").float())
+        self.correction.copy_(get(prefix + "correction").float())
+        for e in range(self.spec.experts):
+            p = f"{prefix}e{e}."
+            self.gate_up[e].copy_(
+                torch.cat([get(p + "gate").to(dt), get(p + "up").to(dt)], dim=0)
+            )
+            self.down[:, e].copy_(get(p + "down").to(dt))
+        if self.shared is not None:
+            self.shared.load(get, prefix + "shared.")
+
+    def _dense(self, h, dense_w, extra):
+        E, ff = self.spec.experts, self.spec.ff
+        T, W = h.shape
+        scaled = scaled_w = None
+        if self.spec.identity:
+            scaled, scaled_w = h, dense_w[:, E:].sum(dim=1)
+        ar = torch.arange(T, dtype=torch.int32, device=h.device)
+        if E == 0:
+            y = torch.zeros((T, W), dtype=h.dtype, device=h.device)
+        else:
+            gu = F.linear(h, self.gate_up.view(E * 2 * ff, W))
+            act = ops.glu_silu_scale(
+                gu.view(T * E, 2 * ff), dense_w[:, :E].reshape(-1)
+            )
+            y = F.linear(act.view(T, E * ff), self.down.view(W, E * ff))
+        return ops.combine_rows(y, ar, 1, extra, None, scaled, scaled_w)
+
+    def _sorted(self, h, idx, w, extra):
+        E, top = self.spec.experts, self.spec.top
+        R = self.spec.router_outputs
+        flat = idx.view(-1).long()
+        order = torch.sort(flat, stable=True).indices
+        counts = torch.bincount(flat, minlength=R).tolist()  # host sync
+        xs = ops.gather_scale_rows(h, (order // top).to(torch.int32))
+        n = xs.shape[0]
+        n_real = sum(counts[:E])
+        gu = torch.empty((n_real, 2 * self.spec.ff), dtype=h.dtype, device=h.device)
+        a = 0
+        for e in range(E):
+            c = counts[e]
+            if c:
+                torch.mm(xs[a : a + c], self.gate_up[e].t(), out=gu[a : a + c])
+            a += c
+        act = ops.glu_silu_scale(gu)
+        # rows of identity experts (sorted last) keep their input
+        ys = xs.clone() if n_real < n else torch.empty_like(xs)
+        a = 0
+        for e in range(E):
+            c = counts[e]
+            if c:
+                torch.mm(act[a : a + c], self.down[:, e].t(), out=ys[a : a + c])
+            a += c
+        # pair p = t*top + k sits at sorted row inv[p]
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(n, device=h.device)
+        return ops.combine_rows(ys, inv.to(torch.int32), top, extra, w.view(-1))
+
+    def forward(self, h):
+        """[T, width] in the activation dtype -> fp32 [T, width]."""
+        T = h.shape[0]
+        extra = self.shared(h) if self.shared is not None else None
+        dense = T <= self.dense_max_tokens or (
+            h.is_cuda and torch.cuda.is_current_stream_capturing()
+        )
+        idx, w, dense_w, _ = ops.route_tokens(
+            h, self.router, self.spec.top, softmax=True, renorm=True,
+            dense=dense, correction=self.correction,
+            renorm_eps=self.RENORM_EPS,
         )
         if dense:
             return self._dense(h, dense_w, extra)

@@ -50,6 +50,12 @@ register(
     "kserve_amd.models.desalix.DesalixForCausalLM",
     ("kserve_amd_seq_C",),
 )
+register(
+    "Voborax",
+    "kserve_amd.engine.config.HybridModelConfig",
+    "kserve_amd.models.voborax.VoboraxForCausalLM",
+    ("kserve_amd_seq_C",),
+)
 
 
 def architecture_of(config_json: dict) -> str:

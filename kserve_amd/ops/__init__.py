@@ -428,13 +428,16 @@ def qk_norm_temp_cache(
 def ctx_attention_f32(
     q, k_cache, v_cache, block_tables, cu_q, ctx_lens, scale: float,
     max_q_len: int, heads: int, gate=None, out_dtype=torch.float32,
-    sink=None, chunk: int = 0, out_inv_freq=None,
+    sink=None, chunk: int = 0, out_inv_freq=None, window: int = 0,
 ):
     """Paged causal attention with fp32 scores and weights. Optional parts:
     ``gate`` [T, heads] (output times sigmoid), ``sink`` [heads] fp32 (one
     more term exp(sink) in the softmax denominator), ``chunk`` (a query sees
-    only keys of its own block of that many positions), ``out_inv_freq``
-    [vdim/2] fp32 (each head output turned back by its query position)."""
+    only keys of its own block of that many positions), ``window`` (a query
+    sees itself and the window-1 positions before it), ``out_inv_freq``
+    [vdim/2] fp32 (each head output turned back by its query position).
+    ``v_cache`` may be a view of the leading columns of ``k_cache`` (values
+    that are a prefix of the keys are stored once)."""
     if q.is_cuda:
         out = torch.empty(
             (q.shape[0], heads * v_cache.shape[3]), dtype=out_dtype,
@@ -443,12 +446,12 @@ def ctx_attention_f32(
         _native_seq("ctx_attention_f32").ctx_attention_f32(
             out, q, k_cache, v_cache, block_tables, cu_q, ctx_lens, gate,
             float(scale), int(max_q_len), int(heads), sink, int(chunk),
-            out_inv_freq,
+            out_inv_freq, int(window),
         )
         return out
     return torch_ref.ctx_attention_f32(
         q, k_cache, v_cache, block_tables, cu_q, ctx_lens, scale, heads,
-        gate, out_dtype, sink, chunk, out_inv_freq,
+        gate, out_dtype, sink, chunk, out_inv_freq, window,
     )
 
 
@@ -498,10 +501,11 @@ def post_norm_add_rms_norm(
 
 def router_topk(
     logits, top: int, softmax: bool = False, renorm: bool = False,
-    dense: bool = False,
+    dense: bool = False, correction=None, renorm_eps: float = 0.0,
 ):
     """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32
-    [T, top], dense [T, E] weights or None) by sigmoid (or softmax) score."""
+    [T, top], dense [T, E] weights or None) by sigmoid (or softmax) score;
+    with ``correction`` [E] fp32 the choice goes by score + correction."""
     if logits.is_cuda:
         T, E = logits.shape
         idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
@@ -511,15 +515,19 @@ def router_topk(
             if dense else None
         )
         _native_seq("router_topk").router_topk(
-            idx, w, dw, logits, bool(softmax), bool(renorm)
+            idx, w, dw, logits, bool(softmax), bool(renorm), correction,
+            float(renorm_eps),
         )
         return idx, w, dw
-    return torch_ref.router_topk(logits, top, softmax, renorm, dense)
+    return torch_ref.router_topk(
+        logits, top, softmax, renorm, dense, correction, renorm_eps
+    )
 
 
 def route_tokens(
     h, router, top: int, softmax: bool = False, renorm: bool = False,
-    dense: bool = False, want_logits: bool = False,
+    dense: bool = False, want_logits: bool = False, correction=None,
+    renorm_eps: float = 0.0,
 ):
     """The router in one kernel: fp32 logits of h [T, W] (activation dtype)
     against fp32 router rows [E, W], scores, the ``top`` experts. Returns
@@ -533,14 +541,19 @@ def route_tokens(
         dw = torch.empty((T, E), dtype=torch.float32, device=dev) if dense else None
         lg = torch.empty((T, E), dtype=torch.float32, device=dev) if want_logits else None
         _native_seq("route_tokens").route_tokens(
-            idx, w, dw, lg, h, router, bool(softmax), bool(renorm)
+            idx, w, dw, lg, h, router, bool(softmax), bool(renorm), correction,
+            float(renorm_eps),
         )
         return idx, w, dw, lg
-    return torch_ref.route_tokens(h, router, top, softmax, renorm, dense, want_logits)
+    return torch_ref.route_tokens(
+        h, router, top, softmax, renorm, dense, want_logits, correction,
+        renorm_eps,
+    )
 
 
-def gather_scale_rows(x, rows, scales):
-    """out[r] = x[rows[r]] * scales[r] in x's dtype (rows int32, scales fp32)."""
+def gather_scale_rows(x, rows, scales=None):
+    """out[r] = x[rows[r]] * scales[r] in x's dtype (rows int32, scales fp32
+    or None for a plain gather)."""
     if x.is_cuda:
         out = torch.empty((rows.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
         _native_seq("gather_scale_rows").gather_scale_rows(out, x, rows, scales)
@@ -548,13 +561,18 @@ def gather_scale_rows(x, rows, scales):
     return torch_ref.gather_scale_rows(x, rows, scales)
 
 
-def combine_rows(y, index, top: int, extra=None):
-    """fp32 out[t] = sum_k y[index[t*top + k]] (+ extra[t])."""
+def combine_rows(
+    y, index, top: int, extra=None, weights=None, scaled=None, scaled_w=None
+):
+    """fp32 out[t] = sum_k weights[t*top + k] * y[index[t*top + k]]
+    (+ extra[t]) (+ scaled_w[t] * scaled[t]); weights (fp32) default to 1."""
     if y.is_cuda:
         out = _f32_like(index.numel() // top, y.shape[1], y)
-        _native_seq("combine_rows").combine_rows(out, y, index, int(top), extra)
+        _native_seq("combine_rows").combine_rows(
+            out, y, index, int(top), extra, weights, scaled, scaled_w
+        )
         return out
-    return torch_ref.combine_rows(y, index, top, extra)
+    return torch_ref.combine_rows(y, index, top, extra, weights, scaled, scaled_w)
 
 
 def clamped_swiglu(x, alpha: float, limit: float):
@@ -567,3 +585,89 @@ def clamped_swiglu(x, alpha: float, limit: float):
         )
         return out
     return torch_ref.clamped_swiglu(x, alpha, limit)
+
+
+# -- latent attention, post-layer-norm residual, plain feed-forwards ----------
+
+def post_layer_norm_add(
+    residual, delta, weight, mult: float, eps: float, out_dtype,
+    next_weight=None, want_out: bool = True,
+):
+    """fp32 residual (in place) += mult * LayerNorm(delta) * weight (no bias)
+    when ``delta`` is given; returns the new residual in ``out_dtype`` or,
+    with ``next_weight``, its layer norm times that weight."""
+    if residual.is_cuda:
+        out = (
+            torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+            if want_out else None
+        )
+        _native_seq("post_layer_norm_add").post_layer_norm_add(
+            residual, delta, weight, float(mult), float(eps), out, next_weight
+        )
+        return out
+    return torch_ref.post_layer_norm_add(
+        residual, delta, weight, mult, eps, out_dtype, next_weight, want_out
+    )
+
+
+def latent_norm_rope_cache(
+    proj, q_rank: int, kv_rank: int, rot_dim: int, qw, kw, positions,
+    slot_mapping, cache, eps: float, inv_freq,
+):
+    """Rows [query latent | kv latent | key part | ...] -> the RMS-normed
+    query latent (returned, activation dtype) and, when ``cache`` is given,
+    [normed kv latent | key part rotated in pairs (2i, 2i+1)] scattered into
+    the paged cache [blocks, 1, block, kv_rank + rot_dim]."""
+    if proj.is_cuda:
+        cq = torch.empty((proj.shape[0], q_rank), dtype=proj.dtype, device=proj.device)
+        _native_seq("latent_norm_rope_cache").latent_norm_rope_cache(
+            cq, proj, int(q_rank), int(kv_rank), int(rot_dim), qw, kw,
+            positions, slot_mapping, cache, float(eps), inv_freq,
+        )
+        return cq
+    return torch_ref.latent_norm_rope_cache(
+        proj, q_rank, kv_rank, rot_dim, qw, kw, positions, slot_mapping,
+        cache, eps, inv_freq,
+    )
+
+
+def head_matmul_rope(
+    x, w, heads: int, tail: int = 0, positions=None, inv_freq=None,
+    out_dtype=None,
+):
+    """Per-head matrix product with an optional rotated tail:
+    x [T, heads*(k + tail)], w [heads, k, n] -> [T, heads*(n + tail)], the
+    tail coordinates turned in pairs by the token's position."""
+    out_dtype = out_dtype or x.dtype
+    if x.is_cuda:
+        n = w.shape[2]
+        out = torch.empty(
+            (x.shape[0], heads * (n + tail)), dtype=out_dtype, device=x.device
+        )
+        _native_seq("head_matmul_rope").head_matmul_rope(
+            out, x, w, int(heads), int(tail), positions, inv_freq
+        )
+        return out
+    return torch_ref.head_matmul_rope(
+        x, w, heads, tail, positions, inv_freq, out_dtype
+    )
+
+
+def glu_silu_scale(x, scales=None):
+    """[rows, 2 d] = [gate | up] -> silu(gate) * up (* scales[row])."""
+    if x.is_cuda:
+        out = torch.empty(
+            (x.shape[0], x.shape[1] // 2), dtype=x.dtype, device=x.device
+        )
+        _native_seq("glu_silu_scale").glu_silu_scale(out, x, scales)
+        return out
+    return torch_ref.glu_silu_scale(x, scales)
+
+
+def bias_gelu_tanh(x, bias):
+    """gelu (tanh form) of x + bias, in x's dtype."""
+    if x.is_cuda:
+        out = torch.empty_like(x)
+        _native_seq("bias_gelu_tanh").bias_gelu_tanh(out, x, bias)
+        return out
+    return torch_ref.bias_gelu_tanh(x, bias)

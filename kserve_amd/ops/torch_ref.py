@@ -438,7 +438,7 @@ def qk_norm_temp_cache(
 def ctx_attention_f32(
     q, k_cache, v_cache, block_tables, cu_q, ctx_lens, scale: float,
     heads: int, gate=None, out_dtype=torch.float32, sink=None, chunk: int = 0,
-    out_inv_freq=None,
+    out_inv_freq=None, window: int = 0,
 ):
     _, G, bs, D = k_cache.shape
     DV = v_cache.shape[3]
@@ -463,6 +463,8 @@ def ctx_attention_f32(
         vis = kpos <= qpos
         if chunk > 0:
             vis = vis & (kpos // chunk == qpos // chunk)
+        if window > 0:
+            vis = vis & (qpos - kpos < window)
         sc = sc.masked_fill(~vis.unsqueeze(0), float("-inf"))
         if sink is None:
             w = torch.softmax(sc, dim=-1)
@@ -558,48 +560,68 @@ def post_norm_add_rms_norm(
 
 def router_topk(
     logits, top: int, softmax: bool = False, renorm: bool = False,
-    dense: bool = False,
+    dense: bool = False, correction=None, renorm_eps: float = 0.0,
 ):
     """Scores (sigmoid, or softmax over the experts) of fp32 router logits
     [T, E]; the ``top`` largest per token -> (indices int32 [T, top],
     weights fp32 [T, top], and with ``dense`` the same weights as a [T, E]
-    matrix that is zero elsewhere), optionally renormalised to sum 1."""
+    matrix that is zero elsewhere), optionally renormalised to sum 1
+    (divided by their sum + ``renorm_eps``). With ``correction`` [E] the
+    choice goes by score + correction while the weights stay the scores."""
     z = logits.float()
     s = torch.softmax(z, dim=-1) if softmax else torch.sigmoid(z)
-    w, idx = s.topk(top, dim=-1)
+    if correction is None:
+        w, idx = s.topk(top, dim=-1)
+    else:
+        idx = (s + correction.float()).topk(top, dim=-1).indices
+        w = torch.gather(s, 1, idx)
     if renorm:
-        w = w / w.sum(-1, keepdim=True)
+        w = w / (w.sum(-1, keepdim=True) + renorm_eps)
     dw = torch.zeros_like(s).scatter_(1, idx, w) if dense else None
     return idx.to(torch.int32), w, dw
 
 
 def route_tokens(
     h, router, top: int, softmax: bool = False, renorm: bool = False,
-    dense: bool = False, want_logits: bool = False,
+    dense: bool = False, want_logits: bool = False, correction=None,
+    renorm_eps: float = 0.0,
 ):
     """Router logits h @ router^T in fp32 (h in the activation dtype, router
     fp32 [E, W]) followed by ``router_topk``; returns (indices, weights,
     dense weights or None, logits or None)."""
     logits = torch.nn.functional.linear(h.float(), router.float())
-    idx, w, dw = router_topk(logits, top, softmax, renorm, dense)
+    idx, w, dw = router_topk(
+        logits, top, softmax, renorm, dense, correction, renorm_eps
+    )
     return idx, w, dw, (logits if want_logits else None)
 
 
 def gather_scale_rows(x, rows, scales):
-    """out[r] = x[rows[r]] * scales[r] (product in fp32, rounded to x's dtype)."""
+    """out[r] = x[rows[r]] * scales[r] (product in fp32, rounded to x's dtype);
+    without scales a plain row gather."""
+    if scales is None:
+        return x[rows.long()].contiguous()
     return (x[rows.long()].float() * scales.float().unsqueeze(1)).to(x.dtype)
 
 
-def combine_rows(y, index, top: int, extra=None):
-    """out[t] = sum_k y[index[t * top + k]] (+ extra[t]), summed in fp32 in
-    the order k = 0..top-1, extra last; fp32 result."""
+def combine_rows(
+    y, index, top: int, extra=None, weights=None, scaled=None, scaled_w=None
+):
+    """out[t] = sum_k weights[t*top + k] * y[index[t*top + k]] (+ extra[t])
+    (+ scaled_w[t] * scaled[t]), summed in fp32 in the order k = 0..top-1,
+    extra, scaled row; weights default to 1; fp32 result."""
     T = index.numel() // top
     out = torch.zeros(T, y.shape[1], dtype=torch.float32, device=y.device)
     idx = index.long().view(T, top)
     for k in range(top):
-        out += y[idx[:, k]].float()
+        r = y[idx[:, k]].float()
+        if weights is not None:
+            r = r * weights.float().view(T, top)[:, k : k + 1]
+        out += r
     if extra is not None:
         out += extra.float()
+    if scaled is not None:
+        out += scaled.float() * scaled_w.float().view(T, 1)
     return out
 
 
@@ -608,3 +630,103 @@ def clamped_swiglu(x, alpha: float, limit: float):
     g = x[..., :d].float().clamp(max=limit)
     u = x[..., d:].float().clamp(-limit, limit)
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(x.dtype)
+
+
+# -- latent attention, post-layer-norm residual, plain feed-forwards ----------
+
+def post_layer_norm_add(
+    residual, delta, weight, mult: float, eps: float, out_dtype,
+    next_weight=None, want_out: bool = True,
+):
+    """residual (fp32, in place) += mult * LayerNorm(delta) * weight (mean
+    removed, biased variance, no bias term), when ``delta`` is given. Returns
+    the new residual in ``out_dtype`` or, with ``next_weight``, its layer
+    norm times that weight (None when ``want_out`` is false)."""
+    if delta is not None:
+        d = delta.float()
+        d = d - d.mean(-1, keepdim=True)
+        d = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps)
+        residual += mult * (d * weight)
+    if not want_out:
+        return None
+    if next_weight is None:
+        return residual.to(out_dtype)
+    r = residual - residual.mean(-1, keepdim=True)
+    r = r * torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + eps)
+    return (r * next_weight).to(out_dtype)
+
+
+def rotate_pairs(x, positions, inv_freq):
+    """Rotate the first 2*len(inv_freq) coordinates of the last axis of
+    x [T, ..., n] (fp32): coordinate 2i pairs with 2i+1 and turns by
+    position * inv_freq[i]; angles and sin/cos in fp32."""
+    half = 0 if inv_freq is None else inv_freq.numel()
+    if half == 0:
+        return x
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
+    a = (positions.to(torch.float32).view(-1, 1) * inv_freq.view(1, -1)).view(shape)
+    c, s = torch.cos(a), torch.sin(a)
+    u, v = x[..., 0 : 2 * half : 2], x[..., 1 : 2 * half : 2]
+    out = x.clone()
+    out[..., 0 : 2 * half : 2] = u * c - v * s
+    out[..., 1 : 2 * half : 2] = v * c + u * s
+    return out
+
+
+def latent_norm_rope_cache(
+    proj, q_rank: int, kv_rank: int, rot_dim: int, qw, kw, positions,
+    slot_mapping, cache, eps: float, inv_freq,
+):
+    """proj [T, >= q_rank + kv_rank + rot_dim] = [query latent | kv latent |
+    key part to rotate | ...]. Returns the RMS-normed query latent times
+    ``qw`` in proj's dtype; writes [normed kv latent * kw | rotated key part]
+    into ``cache`` [blocks, 1, block, kv_rank + rot_dim] at the tokens'
+    slots (negative slots are skipped). ``cache`` None: the query side only."""
+    x = proj[:, :q_rank].float()
+    cq = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * qw
+    if cache is not None:
+        c = proj[:, q_rank : q_rank + kv_rank].float()
+        c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * kw
+        row = c
+        if rot_dim:
+            kr = proj[:, q_rank + kv_rank : q_rank + kv_rank + rot_dim].float()
+            row = torch.cat([c, rotate_pairs(kr, positions, inv_freq)], dim=-1)
+        bs = cache.shape[2]
+        slots = slot_mapping[: proj.shape[0]].long()
+        ok = slots >= 0
+        cache[slots[ok] // bs, 0, slots[ok] % bs] = row[ok].to(cache.dtype)
+    return cq.to(proj.dtype)
+
+
+def head_matmul_rope(
+    x, w, heads: int, tail: int, positions, inv_freq, out_dtype
+):
+    """x [T, heads * (k + tail)], w [heads, k, n] -> [T, heads * (n + tail)]:
+    per head the first k coordinates times the head's matrix (fp32 sums),
+    followed by the ``tail`` coordinates rotated in pairs by the token's
+    position (copied when ``inv_freq`` is None)."""
+    T = x.shape[0]
+    H, k, n = w.shape
+    xh = x.reshape(T, heads, k + tail).float()
+    y = torch.einsum("thk,hkn->thn", xh[..., :k], w.float())
+    if tail:
+        y = torch.cat([y, rotate_pairs(xh[..., k:], positions, inv_freq)], dim=-1)
+    return y.reshape(T, heads * (n + tail)).to(out_dtype)
+
+
+def glu_silu_scale(x, scales=None):
+    """x [rows, 2 d] = [gate | up] -> silu(gate) * up (* scales[row]) in x's
+    dtype; arithmetic in fp32."""
+    d = x.shape[-1] // 2
+    g, u = x[..., :d].float(), x[..., d:].float()
+    y = g * torch.sigmoid(g) * u
+    if scales is not None:
+        y = y * scales.float().view(-1, 1)
+    return y.to(x.dtype)
+
+
+def bias_gelu_tanh(x, bias):
+    """gelu (tanh form) of x + bias in x's dtype; arithmetic in fp32."""
+    z = x.float() + bias.float()
+    y = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
+    return y.to(x.dtype)
