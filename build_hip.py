@@ -47,6 +47,7 @@ MODULES = {
             "residual_norm_f32.hip",
             "ssm_scan.hip",
             "attention_f32.hip",
+            "latent_attention.hip",
             "moe_route.hip",
             "activation.hip",
             "sampling.hip",

@@ -299,7 +299,8 @@ struct TileStage {
 
   __device__ __forceinline__ void fetch(const T* cache, const int* bt, int k0,
                                         int nk, int g, int kv_heads, int W,
-                                        int block_size, int bs_shift, bool vec) {
+                                        long row_stride, int block_size,
+                                        int bs_shift, bool vec) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = threadIdx.x + NT * i;
@@ -311,8 +312,8 @@ struct TileStage {
         const int pb = bs_shift >= 0 ? kp >> bs_shift : kp / block_size;
         const int po = bs_shift >= 0 ? kp & (block_size - 1) : kp % block_size;
         const long blk = bt[pb];
-        ch[i].load(cache + ((blk * kv_heads + g) * block_size + po) * W + d0, vec,
-                   valid);
+        ch[i].load(cache + ((blk * kv_heads + g) * block_size + po) * row_stride + d0,
+                   vec, valid);
       } else {
         ch[i].zero();
       }
@@ -339,7 +340,7 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     const T* __restrict__ gate, long gate_stride, float scale, int heads,
     int kv_heads, int D, int DV, int block_size, int hpb,
     const float* __restrict__ sink, int chunk,
-    const float* __restrict__ out_inv_freq) {
+    const float* __restrict__ out_inv_freq, int window, long v_row_stride) {
   extern __shared__ float lds[];
   constexpr int KS = DP + 4;   // K row stride: lanes of one MFMA read hit 64 banks
   constexpr int VS = DVP + 4;  // V row stride: likewise for the 4-key-apart rows
@@ -373,16 +374,24 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   const int hd = head0 + r % hpb;
   const int qpos = row_ok ? base_pos + r / hpb : -1;
   // first visible key of this lane's query, of the block and of this wave
-  const int qstart = (chunk > 0 && row_ok) ? qpos / chunk * chunk : 0;
-  const int kbeg = chunk > 0 ? base_pos / chunk * chunk : 0;
+  // (chunk and window exclude each other: the host checks)
+  const int qstart = !row_ok      ? 0
+                     : chunk > 0  ? qpos / chunk * chunk
+                     : window > 0 ? max(qpos - window + 1, 0)
+                                  : 0;
+  const int kbeg = chunk > 0    ? base_pos / chunk * chunk
+                   : window > 0 ? max(base_pos - window + 1, 0)
+                                : 0;
   // keys this wave needs: from its first row's chunk up to its own last
   // row's position
   const int wave_last =
       SPLITK ? last_pos : base_pos + min(wave * 16 + 15, nrows - 1) / hpb;
+  const int wave_first_pos = base_pos + min(wave * 16, nrows - 1) / hpb;
   const int wave_first =
-      (SPLITK || chunk <= 0)
-          ? kbeg
-          : (base_pos + min(wave * 16, nrows - 1) / hpb) / chunk * chunk;
+      SPLITK       ? kbeg
+      : chunk > 0  ? wave_first_pos / chunk * chunk
+      : window > 0 ? max(wave_first_pos - window + 1, 0)
+                   : kbeg;
 
   // Q^T fragments (B operand). The contraction over the head dimension may
   // run in any order as long as both operands agree: k-step ks of lane group
@@ -402,7 +411,9 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   float m = -INFINITY, l = 0.f;
 
   const int* bt = block_tables + (long)s * bt_stride;
-  const bool kvec = (D % 8) == 0, vvec = (DV % 8) == 0;
+  const bool kvec = (D % 8) == 0;
+  const bool vvec = (DV % 8) == 0 && (v_row_stride % 8) == 0 &&
+                    ((uintptr_t)v_cache % 32) == 0;
   const int bs_shift =
       (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
   constexpr int KT = SPLITK ? 1 : 4;  // 16-key sub-tiles per wave and tile
@@ -410,8 +421,8 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   // the next tile's global loads are in flight while this one is computed
   TileStage<T, DP> kst;
   TileStage<T, DVP> vst;
-  kst.fetch(k_cache, bt, kbeg, min(BK, last_pos + 1 - kbeg), g, kv_heads, D, block_size, bs_shift, kvec);
-  vst.fetch(v_cache, bt, kbeg, min(BK, last_pos + 1 - kbeg), g, kv_heads, DV, block_size, bs_shift, vvec);
+  kst.fetch(k_cache, bt, kbeg, min(BK, last_pos + 1 - kbeg), g, kv_heads, D, D, block_size, bs_shift, kvec);
+  vst.fetch(v_cache, bt, kbeg, min(BK, last_pos + 1 - kbeg), g, kv_heads, DV, v_row_stride, block_size, bs_shift, vvec);
   for (int k0 = kbeg; k0 <= last_pos; k0 += BK) {
     __syncthreads();  // previous tile fully consumed
     kst.store(Ks);
@@ -419,8 +430,8 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     __syncthreads();
     if (k0 + BK <= last_pos) {
       const int nn = min(BK, last_pos + 1 - (k0 + BK));
-      kst.fetch(k_cache, bt, k0 + BK, nn, g, kv_heads, D, block_size, bs_shift, kvec);
-      vst.fetch(v_cache, bt, k0 + BK, nn, g, kv_heads, DV, block_size, bs_shift, vvec);
+      kst.fetch(k_cache, bt, k0 + BK, nn, g, kv_heads, D, D, block_size, bs_shift, kvec);
+      vst.fetch(v_cache, bt, k0 + BK, nn, g, kv_heads, DV, v_row_stride, block_size, bs_shift, vvec);
     }
     if (k0 > wave_last || k0 + BK <= wave_first) continue;
 
@@ -688,6 +699,7 @@ hipError_t launch_ctx_attention(void* out, const void* q, const void* k_cache,
                                 int max_q_len, int heads, int kv_heads, int D,
                                 int DV, int block_size, const void* sink,
                                 int chunk, const void* out_inv_freq,
+                                int window, long v_row_stride,
                                 hipStream_t stream) {
   size_t smem = sizeof(float) * (size_t)BK * (DP + 4 + DVP + 4);
   const bool decode = max_q_len == 1;
@@ -714,14 +726,15 @@ hipError_t launch_ctx_attention(void* out, const void* q, const void* k_cache,
                      (const int*)block_tables, bt_stride, (const int*)cu_q,
                      (const int*)ctx_lens, (const T*)gate, gate_stride, scale,
                      heads, kv_heads, D, DV, block_size, hpb,
-                     (const float*)sink, chunk, (const float*)out_inv_freq);
+                     (const float*)sink, chunk, (const float*)out_inv_freq,
+                     window, v_row_stride);
   return hipGetLastError();
 }
 
 #define CTX_ARGS                                                              \
   out, q, k_cache, v_cache, block_tables, bt_stride, cu_q, ctx_lens, gate,    \
       gate_stride, scale, num_seqs, max_q_len, heads, kv_heads, D, DV,        \
-      block_size, sink, chunk, out_inv_freq, stream
+      block_size, sink, chunk, out_inv_freq, window, v_row_stride, stream
 
 template <typename T, int DP>
 hipError_t dispatch_dv(void* out, const void* q, const void* k_cache,
@@ -730,8 +743,8 @@ hipError_t dispatch_dv(void* out, const void* q, const void* k_cache,
                        const void* gate, long gate_stride, float scale,
                        int num_seqs, int max_q_len, int heads, int kv_heads,
                        int D, int DV, int block_size, const void* sink,
-                       int chunk, const void* out_inv_freq,
-                       hipStream_t stream) {
+                       int chunk, const void* out_inv_freq, int window,
+                       long v_row_stride, hipStream_t stream) {
   if (DV <= 64) return launch_ctx_attention<T, DP, 64>(CTX_ARGS);
   if (DV <= 128) return launch_ctx_attention<T, DP, 128>(CTX_ARGS);
   return launch_ctx_attention<T, DP, 256>(CTX_ARGS);
@@ -744,8 +757,8 @@ hipError_t dispatch_d(void* out, const void* q, const void* k_cache,
                       const void* gate, long gate_stride, float scale,
                       int num_seqs, int max_q_len, int heads, int kv_heads,
                       int D, int DV, int block_size, const void* sink,
-                      int chunk, const void* out_inv_freq,
-                      hipStream_t stream) {
+                      int chunk, const void* out_inv_freq, int window,
+                      long v_row_stride, hipStream_t stream) {
   if (D <= 64) return dispatch_dv<T, 64>(CTX_ARGS);
   if (D <= 128) return dispatch_dv<T, 128>(CTX_ARGS);
   return dispatch_dv<T, 256>(CTX_ARGS);
@@ -757,10 +770,13 @@ extern "C" hipError_t ks_ctx_attention_f32(
     const void* ctx_lens, const void* gate, long gate_stride, float scale,
     int num_seqs, int max_q_len, int heads, int kv_heads, int D, int DV,
     int block_size, int is_f32, const void* sink, int chunk,
-    const void* out_inv_freq, hipStream_t stream) {
+    const void* out_inv_freq, int window, long v_row_stride,
+    hipStream_t stream) {
   if (num_seqs == 0 || max_q_len == 0) return hipSuccess;
   if (D < 1 || D > 256 || DV < 1 || DV > 256 || kv_heads < 1 ||
-      heads % kv_heads != 0 || chunk < 0 || (out_inv_freq && DV % 2 != 0))
+      heads % kv_heads != 0 || chunk < 0 || window < 0 ||
+      (chunk > 0 && window > 0) || v_row_stride < DV ||
+      (out_inv_freq && DV % 2 != 0))
     return hipErrorInvalidValue;
   return is_f32 ? dispatch_d<float>(CTX_ARGS) : dispatch_d<short>(CTX_ARGS);
 }

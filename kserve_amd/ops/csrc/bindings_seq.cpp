@@ -31,7 +31,7 @@ hipError_t ks_ctx_attention_f32(void*, const void*, const void*, const void*,
                                 const void*, int, const void*, const void*,
                                 const void*, long, float, int, int, int, int,
                                 int, int, int, int, const void*, int,
-                                const void*, hipStream_t);
+                                const void*, int, long, hipStream_t);
 hipError_t ks_qk_headnorm_rope_cache(void*, const void*, const void*,
                                      const void*, long, const void*,
                                      const void*, const void*, const void*,
@@ -43,14 +43,29 @@ hipError_t ks_post_norm_add_rms_norm(void*, const void*, long, int, float,
                                      float, float, void*, int, int, int,
                                      hipStream_t);
 hipError_t ks_router_topk(void*, void*, void*, const void*, int, int, int, int,
-                          int, hipStream_t);
+                          int, const void*, float, hipStream_t);
 hipError_t ks_route_tokens(void*, void*, void*, void*, const void*, long,
-                           const void*, int, int, int, int, int, int, int,
-                           hipStream_t);
+                           const void*, int, int, int, int, int, int,
+                           const void*, float, int, hipStream_t);
 hipError_t ks_gather_scale_rows(void*, const void*, long, const void*,
                                 const void*, int, int, int, hipStream_t);
 hipError_t ks_combine_rows(void*, const void*, const void*, int, const void*,
-                           long, int, int, int, hipStream_t);
+                           long, int, int, int, const void*, const void*, long,
+                           const void*, hipStream_t);
+hipError_t ks_post_layer_norm_add(void*, const void*, long, int, const void*,
+                                  float, float, void*, int, const void*, int,
+                                  int, hipStream_t);
+hipError_t ks_latent_norm_rope_cache(void*, const void*, long, int, int, int,
+                                     int, const void*, const void*,
+                                     const void*, const void*, void*, float,
+                                     const void*, int, int, hipStream_t);
+hipError_t ks_head_matmul_rope(void*, const void*, long, const void*, int, int,
+                               int, int, int, const void*, const void*, int,
+                               int, int, hipStream_t);
+hipError_t ks_glu_silu_scale(void*, const void*, const void*, int, int, int,
+                             hipStream_t);
+hipError_t ks_bias_gelu_tanh(void*, const void*, const void*, int, int, int,
+                             hipStream_t);
 hipError_t ks_clamped_swiglu(void*, const void*, int, int, float, float, int,
                              hipStream_t);
 }
@@ -286,7 +301,8 @@ void ctx_attention_f32(at::Tensor& out, at::Tensor& q, at::Tensor& k_cache,
                        const c10::optional<at::Tensor>& gate, double scale,
                        int64_t max_q_len, int64_t heads,
                        const c10::optional<at::Tensor>& sink, int64_t chunk,
-                       const c10::optional<at::Tensor>& out_inv_freq) {
+                       const c10::optional<at::Tensor>& out_inv_freq,
+                       int64_t window) {
   CHECK_F32(q);
   CHECK_I32(cu_q);
   CHECK_I32(ctx_lens);
@@ -294,12 +310,17 @@ void ctx_attention_f32(at::Tensor& out, at::Tensor& q, at::Tensor& k_cache,
                   block_tables.dim() == 2 && block_tables.stride(1) == 1,
               "block_tables [seqs, blocks] int32");
   TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 &&
-                  k_cache.is_contiguous() && v_cache.is_contiguous() &&
-                  out.is_contiguous(),
+                  k_cache.is_contiguous() && out.is_contiguous(),
               "caches [blocks, kv_heads, block, dim]");
   const int f32 = act_is_f32(out, "out");
   const int G = k_cache.size(1), bs = k_cache.size(2), D = k_cache.size(3);
   const int DV = v_cache.size(3);
+  // the values may be a column range of wider rows (a view of the key pool)
+  const int64_t vrs = v_cache.stride(2);
+  TORCH_CHECK(v_cache.stride(3) == 1 && vrs >= DV &&
+                  v_cache.stride(1) == vrs * bs &&
+                  v_cache.stride(0) == vrs * bs * G,
+              "v_cache: dense pages of rows with one common stride");
   const int num_seqs = ctx_lens.numel();
   const int64_t tokens = q.numel() / (heads * D);
   TORCH_CHECK(act_is_f32(k_cache, "k_cache") == f32 &&
@@ -332,14 +353,15 @@ void ctx_attention_f32(at::Tensor& out, at::Tensor& q, at::Tensor& k_cache,
                 "out_inv_freq [vdim / 2] fp32");
     fp = out_inv_freq->data_ptr();
   }
-  TORCH_CHECK(chunk >= 0, "chunk must not be negative");
+  TORCH_CHECK(chunk >= 0 && window >= 0 && !(chunk > 0 && window > 0),
+              "chunk / window: not negative, at most one of them");
   check_hip(ks_ctx_attention_f32(
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                 v_cache.data_ptr(), block_tables.data_ptr(),
                 (int)block_tables.stride(0), cu_q.data_ptr(),
                 ctx_lens.data_ptr(), gp, gst, (float)scale, num_seqs,
                 (int)max_q_len, (int)heads, G, D, DV, bs, f32, sp, (int)chunk,
-                fp, current_stream()),
+                fp, (int)window, (long)vrs, current_stream()),
             "ctx_attention_f32");
 }
 
@@ -455,7 +477,9 @@ void post_norm_add_rms_norm(at::Tensor& residual,
 
 void router_topk(at::Tensor& idx, at::Tensor& w,
                  const c10::optional<at::Tensor>& dense, at::Tensor& logits,
-                 bool softmax, bool renorm) {
+                 bool softmax, bool renorm,
+                 const c10::optional<at::Tensor>& correction,
+                 double renorm_eps) {
   CHECK_F32(logits);
   CHECK_F32(w);
   CHECK_I32(idx);
@@ -469,16 +493,24 @@ void router_topk(at::Tensor& idx, at::Tensor& w,
     TORCH_CHECK(dense->numel() == logits.numel(), "dense [T, E]");
     dp = dense->data_ptr();
   }
+  const void* cp = nullptr;
+  if (correction.has_value()) {
+    CHECK_F32(*correction);
+    TORCH_CHECK(correction->numel() == E, "correction [E]");
+    cp = correction->data_ptr();
+  }
   check_hip(ks_router_topk(idx.data_ptr(), w.data_ptr(), dp, logits.data_ptr(),
-                           T, E, top, softmax ? 1 : 0, renorm ? 1 : 0,
-                           current_stream()),
+                           T, E, top, softmax ? 1 : 0, renorm ? 1 : 0, cp,
+                           (float)renorm_eps, current_stream()),
             "router_topk");
 }
 
 void route_tokens(at::Tensor& idx, at::Tensor& w,
                   const c10::optional<at::Tensor>& dense,
                   const c10::optional<at::Tensor>& logits_out, at::Tensor& h,
-                  at::Tensor& router, bool softmax, bool renorm) {
+                  at::Tensor& router, bool softmax, bool renorm,
+                  const c10::optional<at::Tensor>& correction,
+                  double renorm_eps) {
   CHECK_ROWS(h);
   CHECK_F32(router);
   CHECK_F32(w);
@@ -500,32 +532,46 @@ void route_tokens(at::Tensor& idx, at::Tensor& w,
     TORCH_CHECK(logits_out->numel() == (int64_t)T * E, "logits [T, E]");
     lp = logits_out->data_ptr();
   }
+  const void* cp = nullptr;
+  if (correction.has_value()) {
+    CHECK_F32(*correction);
+    TORCH_CHECK(correction->numel() == E, "correction [E]");
+    cp = correction->data_ptr();
+  }
   check_hip(ks_route_tokens(idx.data_ptr(), w.data_ptr(), dp, lp, h.data_ptr(),
                             h.stride(0), router.data_ptr(), T, W, E, top,
-                            softmax ? 1 : 0, renorm ? 1 : 0,
-                            act_is_f32(h, "h"), current_stream()),
+                            softmax ? 1 : 0, renorm ? 1 : 0, cp,
+                            (float)renorm_eps, act_is_f32(h, "h"),
+                            current_stream()),
             "route_tokens");
 }
 
 void gather_scale_rows(at::Tensor& out, at::Tensor& x, at::Tensor& rows,
-                       at::Tensor& scales) {
+                       const c10::optional<at::Tensor>& scales) {
   CHECK_ROWS(x);
   CHECK_I32(rows);
-  CHECK_F32(scales);
   const int f32 = act_is_f32(x, "x");
   TORCH_CHECK(out.is_contiguous() && act_is_f32(out, "out") == f32 &&
-                  out.numel() == rows.numel() * x.size(1) &&
-                  scales.numel() == rows.numel(),
+                  out.numel() == rows.numel() * x.size(1),
               "gather_scale_rows: dtype/shape mismatch");
+  const void* scp = nullptr;
+  if (scales.has_value()) {
+    CHECK_F32(*scales);
+    TORCH_CHECK(scales->numel() == rows.numel(), "scales [rows]");
+    scp = scales->data_ptr();
+  }
   check_hip(ks_gather_scale_rows(out.data_ptr(), x.data_ptr(), x.stride(0),
-                                 rows.data_ptr(), scales.data_ptr(),
+                                 rows.data_ptr(), scp,
                                  (int)rows.numel(), (int)x.size(1), f32,
                                  current_stream()),
             "gather_scale_rows");
 }
 
 void combine_rows(at::Tensor& out, at::Tensor& y, at::Tensor& index,
-                  int64_t top, const c10::optional<at::Tensor>& extra) {
+                  int64_t top, const c10::optional<at::Tensor>& extra,
+                  const c10::optional<at::Tensor>& weights,
+                  const c10::optional<at::Tensor>& scaled,
+                  const c10::optional<at::Tensor>& scaled_w) {
   CHECK_F32(out);
   CHECK_I32(index);
   TORCH_CHECK(y.dim() == 2 && y.is_contiguous() && top > 0 &&
@@ -544,9 +590,28 @@ void combine_rows(at::Tensor& out, at::Tensor& y, at::Tensor& index,
     ep = extra->data_ptr();
     est = extra->stride(0);
   }
+  const void *wp = nullptr, *sp = nullptr, *swp = nullptr;
+  long sst = 0;
+  if (weights.has_value()) {
+    CHECK_F32(*weights);
+    TORCH_CHECK(weights->numel() == index.numel(), "weights [T * top]");
+    wp = weights->data_ptr();
+  }
+  if (scaled.has_value()) {
+    CHECK_ROWS(*scaled);
+    TORCH_CHECK(scaled_w.has_value(), "scaled rows need their weights");
+    CHECK_F32(*scaled_w);
+    TORCH_CHECK(act_is_f32(*scaled, "scaled") == f32 &&
+                    scaled->size(0) == tokens && scaled->size(1) == width &&
+                    scaled_w->numel() == tokens,
+                "scaled [T, W] in y's dtype, scaled_w [T]");
+    sp = scaled->data_ptr();
+    sst = scaled->stride(0);
+    swp = scaled_w->data_ptr();
+  }
   check_hip(ks_combine_rows(out.data_ptr(), y.data_ptr(), index.data_ptr(),
-                            (int)top, ep, est, tokens, width, f32,
-                            current_stream()),
+                            (int)top, ep, est, tokens, width, f32, wp, sp, sst,
+                            swp, current_stream()),
             "combine_rows");
 }
 
@@ -563,6 +628,163 @@ void clamped_swiglu(at::Tensor& out, at::Tensor& input, double alpha,
                               (float)alpha, (float)limit, f32,
                               current_stream()),
             "clamped_swiglu");
+}
+
+void post_layer_norm_add(at::Tensor& residual,
+                         const c10::optional<at::Tensor>& delta,
+                         const c10::optional<at::Tensor>& weight, double mult,
+                         double eps, const c10::optional<at::Tensor>& out,
+                         const c10::optional<at::Tensor>& next_weight) {
+  CHECK_F32(residual);
+  TORCH_CHECK(residual.dim() == 2, "residual [T, W]");
+  const int rows = residual.size(0), width = residual.size(1);
+  const void *dp = nullptr, *wp = nullptr, *np = nullptr;
+  void* op = nullptr;
+  long dst = 0;
+  int d_f32 = 1, o_f32 = 1;
+  if (delta.has_value()) {
+    CHECK_ROWS(*delta);
+    TORCH_CHECK(weight.has_value(), "delta needs a norm weight");
+    CHECK_F32(*weight);
+    TORCH_CHECK(delta->size(0) == rows && delta->size(1) == width &&
+                    weight->numel() == width,
+                "delta / weight: shape mismatch");
+    d_f32 = act_is_f32(*delta, "delta");
+    dp = delta->data_ptr();
+    dst = delta->stride(0);
+    wp = weight->data_ptr();
+  }
+  if (next_weight.has_value()) {
+    CHECK_F32(*next_weight);
+    TORCH_CHECK(next_weight->numel() == width, "next_weight [W]");
+    np = next_weight->data_ptr();
+  }
+  if (out.has_value()) {
+    TORCH_CHECK(out->is_contiguous() && out->numel() == residual.numel(),
+                "out [T, W]");
+    o_f32 = act_is_f32(*out, "out");
+    op = out->data_ptr();
+  }
+  check_hip(ks_post_layer_norm_add(residual.data_ptr(), dp, dst, d_f32, wp,
+                                   (float)mult, (float)eps, op, o_f32, np, rows,
+                                   width, current_stream()),
+            "post_layer_norm_add");
+}
+
+void latent_norm_rope_cache(at::Tensor& cq_out, at::Tensor& proj,
+                            int64_t q_rank, int64_t kv_rank, int64_t rot_dim,
+                            at::Tensor& qw,
+                            const c10::optional<at::Tensor>& kw,
+                            at::Tensor& positions, at::Tensor& slot_mapping,
+                            const c10::optional<at::Tensor>& cache, double eps,
+                            const c10::optional<at::Tensor>& inv_freq) {
+  CHECK_ROWS(proj);
+  CHECK_F32(qw);
+  CHECK_I64(positions);
+  CHECK_I32(slot_mapping);
+  const int f32 = act_is_f32(proj, "proj");
+  const int tokens = proj.size(0);
+  TORCH_CHECK(q_rank >= 1 && kv_rank >= 0 && rot_dim >= 0 &&
+                  proj.size(1) >= q_rank + kv_rank + rot_dim &&
+                  qw.numel() == q_rank && cq_out.is_contiguous() &&
+                  act_is_f32(cq_out, "cq_out") == f32 &&
+                  cq_out.numel() == (int64_t)tokens * q_rank &&
+                  positions.numel() >= tokens,
+              "latent_norm_rope_cache: dtype/shape mismatch");
+  const void *kp = nullptr, *fp = nullptr;
+  void* cp = nullptr;
+  int half = 0;
+  if (cache.has_value()) {
+    TORCH_CHECK(kw.has_value(), "a cache needs the kv norm weight");
+    CHECK_F32(*kw);
+    TORCH_CHECK(cache->dim() == 4 && cache->is_contiguous() &&
+                    cache->size(1) == 1 &&
+                    cache->size(3) == kv_rank + rot_dim && kv_rank >= 1 &&
+                    act_is_f32(*cache, "cache") == f32 &&
+                    kw->numel() == kv_rank && slot_mapping.numel() >= tokens,
+                "cache [blocks, 1, block, kv_rank + rot_dim] in proj's dtype");
+    cp = cache->data_ptr();
+    kp = kw->data_ptr();
+    if (inv_freq.has_value()) {
+      CHECK_F32(*inv_freq);
+      half = inv_freq->numel();
+      TORCH_CHECK(2 * half <= rot_dim, "more rotated pairs than the key part has");
+      fp = inv_freq->data_ptr();
+    }
+  }
+  check_hip(ks_latent_norm_rope_cache(
+                cq_out.data_ptr(), proj.data_ptr(), proj.stride(0), tokens,
+                (int)q_rank, (int)kv_rank, (int)rot_dim, qw.data_ptr(), kp,
+                positions.data_ptr(), slot_mapping.data_ptr(), cp, (float)eps,
+                fp, half, f32, current_stream()),
+            "latent_norm_rope_cache");
+}
+
+void head_matmul_rope(at::Tensor& out, at::Tensor& x, at::Tensor& w,
+                      int64_t heads, int64_t tail,
+                      const c10::optional<at::Tensor>& positions,
+                      const c10::optional<at::Tensor>& inv_freq) {
+  CHECK_ROWS(x);
+  TORCH_CHECK(w.dim() == 3 && w.is_contiguous() && w.size(0) == heads,
+              "w [heads, k, n] contiguous");
+  const int in_f32 = act_is_f32(x, "x"), out_f32 = act_is_f32(out, "out");
+  const int tokens = x.size(0), K = w.size(1), N = w.size(2);
+  TORCH_CHECK(act_is_f32(w, "w") == in_f32 && (out_f32 || !in_f32) &&
+                  tail >= 0 && x.size(1) == heads * (K + tail) &&
+                  out.is_contiguous() &&
+                  out.numel() == (int64_t)tokens * heads * (N + tail),
+              "head_matmul_rope: dtype/shape mismatch");
+  const void *pp = nullptr, *fp = nullptr;
+  int half = 0;
+  if (tail > 0 && inv_freq.has_value()) {
+    TORCH_CHECK(positions.has_value(), "rotation needs positions");
+    CHECK_I64(*positions);
+    CHECK_F32(*inv_freq);
+    half = inv_freq->numel();
+    TORCH_CHECK(2 * half <= tail && positions->numel() >= tokens,
+                "more rotated pairs than the tail has / too few positions");
+    pp = positions->data_ptr();
+    fp = inv_freq->data_ptr();
+  }
+  check_hip(ks_head_matmul_rope(out.data_ptr(), x.data_ptr(), x.stride(0),
+                                w.data_ptr(), tokens, (int)heads, K, N,
+                                (int)tail, pp, fp, half, in_f32, out_f32,
+                                current_stream()),
+            "head_matmul_rope");
+}
+
+void glu_silu_scale(at::Tensor& out, at::Tensor& input,
+                    const c10::optional<at::Tensor>& scales) {
+  TORCH_CHECK(input.dim() == 2 && input.is_contiguous() && out.is_contiguous(),
+              "input [rows, 2 d] contiguous");
+  const int rows = input.size(0), d = input.size(1) / 2;
+  const int f32 = act_is_f32(input, "input");
+  TORCH_CHECK(act_is_f32(out, "out") == f32 && input.size(1) == 2 * d &&
+                  out.numel() == (int64_t)rows * d,
+              "glu_silu_scale: dtype/shape mismatch");
+  const void* sp = nullptr;
+  if (scales.has_value()) {
+    CHECK_F32(*scales);
+    TORCH_CHECK(scales->numel() == rows, "scales [rows]");
+    sp = scales->data_ptr();
+  }
+  check_hip(ks_glu_silu_scale(out.data_ptr(), input.data_ptr(), sp, rows, d,
+                              f32, current_stream()),
+            "glu_silu_scale");
+}
+
+void bias_gelu_tanh(at::Tensor& out, at::Tensor& input, at::Tensor& bias) {
+  TORCH_CHECK(input.dim() == 2 && input.is_contiguous() && out.is_contiguous(),
+              "input [rows, d] contiguous");
+  CHECK_F32(bias);
+  const int rows = input.size(0), d = input.size(1);
+  const int f32 = act_is_f32(input, "input");
+  TORCH_CHECK(act_is_f32(out, "out") == f32 && out.numel() == input.numel() &&
+                  bias.numel() == d,
+              "bias_gelu_tanh: dtype/shape mismatch");
+  check_hip(ks_bias_gelu_tanh(out.data_ptr(), input.data_ptr(), bias.data_ptr(),
+                              rows, d, f32, current_stream()),
+            "bias_gelu_tanh");
 }
 
 }  // namespace
@@ -591,5 +813,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "fp32 router logits + sigmoid/softmax scores + top-k experts, fused");
   m.def("gather_scale_rows", &gather_scale_rows, "out[r] = x[rows[r]] * scales[r]");
   m.def("combine_rows", &combine_rows, "fp32 sum of indexed rows per token");
+  m.def("post_layer_norm_add", &post_layer_norm_add,
+        "fp32 residual += mult * LayerNorm(delta) * w, then cast or final layer norm");
+  m.def("latent_norm_rope_cache", &latent_norm_rope_cache,
+        "RMS norm of query / kv latents, pair rotation of the key part, page scatter");
+  m.def("head_matmul_rope", &head_matmul_rope,
+        "per-head matrix product with an optional pair-rotated tail");
+  m.def("glu_silu_scale", &glu_silu_scale, "silu(gate) * up * row scale");
+  m.def("bias_gelu_tanh", &bias_gelu_tanh, "gelu (tanh form) of x + bias");
   def_sampling(m);
 }

@@ -2,7 +2,9 @@
 //
 //  * router_topk: one wave per token. Scores of fp32 logits [T, E] (sigmoid,
 //    or softmax over the experts), the `top` largest chosen one at a time
-//    (ties go to the lower expert), optionally renormalised to sum 1.
+//    (ties go to the lower expert), optionally renormalised to sum 1
+//    (divided by their sum + renorm_eps). With a correction vector the
+//    choice goes by score + correction[e] while the weights stay the scores.
 //    Outputs expert ids and weights [T, top] and, if asked, the same weights
 //    as a dense [T, E] matrix that is zero for experts not chosen.
 //  * route_tokens: the router's matrix product fused in front of the same
@@ -10,9 +12,12 @@
 //    rows, fp32 sums; the logits never travel through memory.
 //  * gather_scale_rows: out[r] = x[rows[r]] * scales[r], product in fp32,
 //    rounded to the activation dtype (an expert's input is the token's input
-//    times its routing weight).
-//  * combine_rows: out[t] = sum_k y[index[t*top + k]] (+ extra[t]) in fp32, k
-//    in ascending order and extra last: no atomics, the same sum every run.
+//    times its routing weight); without scales a plain row gather.
+//  * combine_rows: out[t] = sum_k weights[t*top + k] * y[index[t*top + k]]
+//    (+ extra[t]) (+ scaled_w[t] * scaled[t]) in fp32, k in ascending order,
+//    then extra, then the scaled row: no atomics, the same sum every run.
+//    Weights default to 1; the scaled row is how experts that return their
+//    input join the sum.
 #include "dtype_io.h"
 
 namespace {
@@ -27,7 +32,9 @@ __device__ __forceinline__ void wave_topk(int* __restrict__ idx_out,
                                           float* __restrict__ w_out,
                                           float* __restrict__ dense_out,
                                           const float* z, long t, int E,
-                                          int top, int softmax, int renorm) {
+                                          int top, int softmax, int renorm,
+                                          const float* __restrict__ correction,
+                                          float renorm_eps) {
   const int lane = threadIdx.x & 63;
   float sc[MAX_PER_LANE];  // scores of experts lane + 64 j
   float mx = -INFINITY;
@@ -58,35 +65,42 @@ __device__ __forceinline__ void wave_topk(int* __restrict__ idx_out,
   int my_e = 0;
   float total = 0.f;
   for (int k = 0; k < top; ++k) {
-    float bv = -INFINITY;
+    float bv = -INFINITY;  // choice value (score + correction)
+    float bs = 0.f;        // the score itself
     int be = 0x7fffffff;
 #pragma unroll
     for (int j = 0; j < MAX_PER_LANE; ++j) {
       const int e = lane + 64 * j;
-      if (e < E && !(chosen >> j & 1u) && (sc[j] > bv)) {
-        bv = sc[j];
-        be = e;
+      if (e < E && !(chosen >> j & 1u)) {
+        const float cv = correction ? sc[j] + correction[e] : sc[j];
+        if (cv > bv) {
+          bv = cv;
+          bs = sc[j];
+          be = e;
+        }
       }
     }
     // a lane whose candidates are all taken (or NaN) offers nothing
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
       const float ov = __shfl_xor(bv, off, WAVE_SIZE);
+      const float os = __shfl_xor(bs, off, WAVE_SIZE);
       const int oe = __shfl_xor(be, off, WAVE_SIZE);
       if (ov > bv || (ov == bv && oe < be)) {
         bv = ov;
+        bs = os;
         be = oe;
       }
     }
     if (be == 0x7fffffff) be = 0;  // nothing comparable left (NaN scores)
     if ((be & 63) == lane) chosen |= 1u << (be >> 6);
-    total += bv;
+    total += bs;
     if (lane == k) {
-      my_w = bv;
+      my_w = bs;
       my_e = be;
     }
   }
-  const float norm = renorm ? 1.0f / total : 1.0f;
+  const float norm = renorm ? 1.0f / (total + renorm_eps) : 1.0f;
   if (lane < top) {
     idx_out[t * top + lane] = my_e;
     w_out[t * top + lane] = my_w * norm;
@@ -104,11 +118,13 @@ __global__ void router_topk_kernel(int* __restrict__ idx_out,
                                    float* __restrict__ w_out,
                                    float* __restrict__ dense_out,
                                    const float* __restrict__ logits, int tokens,
-                                   int E, int top, int softmax, int renorm) {
+                                   int E, int top, int softmax, int renorm,
+                                   const float* __restrict__ correction,
+                                   float renorm_eps) {
   const long t = (long)blockIdx.x * NW + (threadIdx.x >> 6);
   if (t >= tokens) return;  // whole waves leave together
   wave_topk(idx_out, w_out, dense_out, logits + t * E, t, E, top, softmax,
-            renorm);
+            renorm, correction, renorm_eps);
 }
 
 // Router logits and the choice in one kernel: a block per token keeps the
@@ -119,7 +135,8 @@ __global__ void __launch_bounds__(NT) route_tokens_kernel(
     int* __restrict__ idx_out, float* __restrict__ w_out,
     float* __restrict__ dense_out, float* __restrict__ logits_out,
     const T* __restrict__ h, long h_stride, const float* __restrict__ router,
-    int W, int E, int top, int softmax, int renorm) {
+    int W, int E, int top, int softmax, int renorm,
+    const float* __restrict__ correction, float renorm_eps) {
   extern __shared__ float lds[];
   float* row = lds;      // [W]
   float* z = lds + ((W + 3) & ~3);  // [E]
@@ -170,7 +187,8 @@ __global__ void __launch_bounds__(NT) route_tokens_kernel(
   }
   __syncthreads();
   if (wave == 0)
-    wave_topk(idx_out, w_out, dense_out, z, t, E, top, softmax, renorm);
+    wave_topk(idx_out, w_out, dense_out, z, t, E, top, softmax, renorm,
+              correction, renorm_eps);
 }
 
 __device__ __forceinline__ void ld4_any(const short* p, float* v) {
@@ -192,6 +210,10 @@ __global__ void gather_scale_rows_kernel(T* __restrict__ out,
                                          int width) {
   const long r = blockIdx.x;
   const T* src = x + (long)rows[r] * x_stride;
+  if (!scales) {
+    for (int i = threadIdx.x; i < width; i += NT) out[r * width + i] = src[i];
+    return;
+  }
   const float s = scales[r];
   for (int i = threadIdx.x; i < width; i += NT)
     st_f32(out, r * width + i, ld_f32(src, i) * s);
@@ -202,11 +224,17 @@ __global__ void combine_rows_kernel(float* __restrict__ out,
                                     const T* __restrict__ y,
                                     const int* __restrict__ index, int top,
                                     const T* __restrict__ extra,
-                                    long extra_stride, int width) {
+                                    long extra_stride, int width,
+                                    const float* __restrict__ weights,
+                                    const T* __restrict__ scaled,
+                                    long scaled_stride,
+                                    const float* __restrict__ scaled_w) {
   const long t = blockIdx.x;
   const bool vec = (width % 4) == 0 && (extra_stride % 4) == 0 &&
+                   (scaled_stride % 4) == 0 &&
                    ((uintptr_t)y % (4 * sizeof(T))) == 0 &&
                    ((uintptr_t)extra % (4 * sizeof(T))) == 0 &&
+                   ((uintptr_t)scaled % (4 * sizeof(T))) == 0 &&
                    ((uintptr_t)out % 16) == 0;
   if (vec) {
     for (int i = threadIdx.x * 4; i < width; i += NT * 4) {
@@ -214,14 +242,22 @@ __global__ void combine_rows_kernel(float* __restrict__ out,
       for (int k = 0; k < top; ++k) {
         float x[4];
         ld4_any(y + (long)index[t * top + k] * width + i, x);
+        const float wk = weights ? weights[t * top + k] : 1.0f;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[c] += x[c];
+        for (int c = 0; c < 4; ++c) acc[c] += wk * x[c];
       }
       if (extra) {
         float x[4];
         ld4_any(extra + t * extra_stride + i, x);
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[c] += x[c];
+      }
+      if (scaled) {
+        float x[4];
+        ld4_any(scaled + t * scaled_stride + i, x);
+        const float ws = scaled_w[t];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[c] += ws * x[c];
       }
       *reinterpret_cast<float4_t*>(out + t * width + i) =
           float4_t{acc[0], acc[1], acc[2], acc[3]};
@@ -231,8 +267,10 @@ __global__ void combine_rows_kernel(float* __restrict__ out,
   for (int i = threadIdx.x; i < width; i += NT) {
     float acc = 0.f;
     for (int k = 0; k < top; ++k)
-      acc += ld_f32(y, (long)index[t * top + k] * width + i);
+      acc += (weights ? weights[t * top + k] : 1.0f) *
+             ld_f32(y, (long)index[t * top + k] * width + i);
     if (extra) acc += ld_f32(extra, t * extra_stride + i);
+    if (scaled) acc += scaled_w[t] * ld_f32(scaled, t * scaled_stride + i);
     out[t * width + i] = acc;
   }
 }
@@ -242,13 +280,15 @@ __global__ void combine_rows_kernel(float* __restrict__ out,
 extern "C" hipError_t ks_router_topk(void* idx_out, void* w_out,
                                      void* dense_out, const void* logits,
                                      int tokens, int E, int top, int softmax,
-                                     int renorm, hipStream_t stream) {
+                                     int renorm, const void* correction,
+                                     float renorm_eps, hipStream_t stream) {
   if (tokens == 0) return hipSuccess;
   if (E < 1 || E > 64 * MAX_PER_LANE || top < 1 || top > E || top > 64)
     return hipErrorInvalidValue;
   hipLaunchKernelGGL(router_topk_kernel, dim3(cdiv(tokens, NW)), dim3(NT), 0,
                      stream, (int*)idx_out, (float*)w_out, (float*)dense_out,
-                     (const float*)logits, tokens, E, top, softmax, renorm);
+                     (const float*)logits, tokens, E, top, softmax, renorm,
+                     (const float*)correction, renorm_eps);
   HIP_CHECK_KERNEL();
   return hipSuccess;
 }
@@ -258,6 +298,7 @@ extern "C" hipError_t ks_route_tokens(void* idx_out, void* w_out,
                                       const void* h, long h_stride,
                                       const void* router, int tokens, int W,
                                       int E, int top, int softmax, int renorm,
+                                      const void* correction, float renorm_eps,
                                       int is_f32, hipStream_t stream) {
   if (tokens == 0) return hipSuccess;
   if (E < 1 || E > 64 * MAX_PER_LANE || top < 1 || top > E || top > 64 ||
@@ -274,7 +315,8 @@ extern "C" hipError_t ks_route_tokens(void* idx_out, void* w_out,
     hipLaunchKernelGGL(route_tokens_kernel<float>, dim3(tokens), dim3(NT), smem,
                        stream, (int*)idx_out, (float*)w_out, (float*)dense_out,
                        (float*)logits_out, (const float*)h, h_stride,
-                       (const float*)router, W, E, top, softmax, renorm);
+                       (const float*)router, W, E, top, softmax, renorm,
+                       (const float*)correction, renorm_eps);
   } else {
     if (smem > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(
@@ -285,7 +327,8 @@ extern "C" hipError_t ks_route_tokens(void* idx_out, void* w_out,
     hipLaunchKernelGGL(route_tokens_kernel<short>, dim3(tokens), dim3(NT), smem,
                        stream, (int*)idx_out, (float*)w_out, (float*)dense_out,
                        (float*)logits_out, (const short*)h, h_stride,
-                       (const float*)router, W, E, top, softmax, renorm);
+                       (const float*)router, W, E, top, softmax, renorm,
+                       (const float*)correction, renorm_eps);
   }
   HIP_CHECK_KERNEL();
   return hipSuccess;
@@ -313,16 +356,23 @@ extern "C" hipError_t ks_combine_rows(void* out, const void* y,
                                       const void* index, int top,
                                       const void* extra, long extra_stride,
                                       int tokens, int width, int is_f32,
+                                      const void* weights, const void* scaled,
+                                      long scaled_stride, const void* scaled_w,
                                       hipStream_t stream) {
   if (tokens == 0) return hipSuccess;
+  if (scaled && !scaled_w) return hipErrorInvalidValue;
   if (is_f32)
     hipLaunchKernelGGL(combine_rows_kernel<float>, dim3(tokens), dim3(NT), 0,
                        stream, (float*)out, (const float*)y, (const int*)index,
-                       top, (const float*)extra, extra_stride, width);
+                       top, (const float*)extra, extra_stride, width,
+                       (const float*)weights, (const float*)scaled,
+                       scaled_stride, (const float*)scaled_w);
   else
     hipLaunchKernelGGL(combine_rows_kernel<short>, dim3(tokens), dim3(NT), 0,
                        stream, (float*)out, (const short*)y, (const int*)index,
-                       top, (const short*)extra, extra_stride, width);
+                       top, (const short*)extra, extra_stride, width,
+                       (const float*)weights, (const short*)scaled,
+                       scaled_stride, (const float*)scaled_w);
   HIP_CHECK_KERNEL();
   return hipSuccess;
 }

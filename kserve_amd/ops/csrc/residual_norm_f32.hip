@@ -11,6 +11,11 @@
 //    += an optional per-token row and an optional shared row, then
 //    out = residual / rms(residual) * next_gain. Both norms have ONE gain for
 //    all channels (host scalars).
+//  * post_layer_norm_add: residual += mult * LayerNorm(delta) * weight (mean
+//    removed, biased variance, no bias term: the norm sits on the sublayer's
+//    OUTPUT), then either out = residual in the activation dtype (the next
+//    sublayer reads the stream itself) or out = LayerNorm(residual) *
+//    next_weight (the model's final norm). Variances are two-pass.
 //  * gated_group_rms_norm: v = y * silu(z), normalised separately in equal
 //    contiguous groups of the row, times a weight (gate before the norm).
 //
@@ -148,6 +153,156 @@ __global__ void add_rms_norm_f32res_vec4_kernel(
       ld4<float>(weight + i, w);
 #pragma unroll
       for (int j = 0; j < 4; ++j) o[j] = keep[k][j] * inv * (w_offset + w[j]);
+      st4<TO>(out + row * width + i, o);
+    }
+  }
+}
+
+template <typename TD, typename TO>
+__global__ void post_layer_norm_add_kernel(
+    float* __restrict__ residual, const TD* __restrict__ delta,
+    long delta_stride, const float* __restrict__ weight, float mult, float eps,
+    TO* __restrict__ out, const float* __restrict__ next_weight, int width) {
+  __shared__ float scratch[NW];
+  const long row = blockIdx.x;
+  float* r = residual + row * width;
+  const float inv_w = 1.0f / (float)width;
+  if (delta) {
+    const TD* d = delta + row * delta_stride;
+    float sm = 0.f;
+    for (int i = threadIdx.x; i < width; i += NT) sm += ld_f32(d, i);
+    const float mean = block_sum_sync<NW>(sm, scratch) * inv_w;
+    float sv = 0.f;
+    for (int i = threadIdx.x; i < width; i += NT) {
+      const float c = ld_f32(d, i) - mean;
+      sv += c * c;
+    }
+    sv = block_sum_sync<NW>(sv, scratch);
+    const float inv = 1.0f / sqrtf(sv * inv_w + eps);
+    for (int i = threadIdx.x; i < width; i += NT)
+      r[i] += mult * ((ld_f32(d, i) - mean) * inv * weight[i]);
+  }
+  if (!out) return;
+  // each thread re-reads only what it wrote itself
+  if (!next_weight) {
+    for (int i = threadIdx.x; i < width; i += NT)
+      st_f32(out, row * width + i, r[i]);
+    return;
+  }
+  float sm = 0.f;
+  for (int i = threadIdx.x; i < width; i += NT) sm += r[i];
+  const float mean = block_sum_sync<NW>(sm, scratch) * inv_w;
+  float sv = 0.f;
+  for (int i = threadIdx.x; i < width; i += NT) {
+    const float c = r[i] - mean;
+    sv += c * c;
+  }
+  sv = block_sum_sync<NW>(sv, scratch);
+  const float inv = 1.0f / sqrtf(sv * inv_w + eps);
+  for (int i = threadIdx.x; i < width; i += NT)
+    st_f32(out, row * width + i, (r[i] - mean) * inv * next_weight[i]);
+}
+
+// the row stays in registers between the passes
+template <typename TD, typename TO>
+__global__ void post_layer_norm_add_vec4_kernel(
+    float* __restrict__ residual, const TD* __restrict__ delta,
+    long delta_stride, const float* __restrict__ weight, float mult, float eps,
+    TO* __restrict__ out, const float* __restrict__ next_weight, int width) {
+  __shared__ float scratch[NW];
+  const long row = blockIdx.x;
+  float* r = residual + row * width;
+  const float inv_w = 1.0f / (float)width;
+  float keep[VEC_STEPS][4];
+  if (delta) {
+    float sm = 0.f;
+#pragma unroll
+    for (int k = 0; k < VEC_STEPS; ++k) {
+      const int i = (threadIdx.x + NT * k) * 4;
+      if (i < width) {
+        ld4<TD>(delta + row * delta_stride + i, keep[k]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sm += keep[k][j];
+      }
+    }
+    const float mean = block_sum_sync<NW>(sm, scratch) * inv_w;
+    float sv = 0.f;
+#pragma unroll
+    for (int k = 0; k < VEC_STEPS; ++k) {
+      const int i = (threadIdx.x + NT * k) * 4;
+      if (i < width) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          keep[k][j] -= mean;
+          sv += keep[k][j] * keep[k][j];
+        }
+      }
+    }
+    sv = block_sum_sync<NW>(sv, scratch);
+    const float inv = 1.0f / sqrtf(sv * inv_w + eps);
+#pragma unroll
+    for (int k = 0; k < VEC_STEPS; ++k) {
+      const int i = (threadIdx.x + NT * k) * 4;
+      if (i < width) {
+        float v[4], w[4];
+        ld4<float>(r + i, v);
+        ld4<float>(weight + i, w);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[j] += mult * (keep[k][j] * inv * w[j]);
+          keep[k][j] = v[j];
+        }
+        st4<float>(r + i, v);
+      }
+    }
+  } else if (out) {
+#pragma unroll
+    for (int k = 0; k < VEC_STEPS; ++k) {
+      const int i = (threadIdx.x + NT * k) * 4;
+      if (i < width) ld4<float>(r + i, keep[k]);
+    }
+  }
+  if (!out) return;
+  if (!next_weight) {
+#pragma unroll
+    for (int k = 0; k < VEC_STEPS; ++k) {
+      const int i = (threadIdx.x + NT * k) * 4;
+      if (i < width) st4<TO>(out + row * width + i, keep[k]);
+    }
+    return;
+  }
+  float sm = 0.f;
+#pragma unroll
+  for (int k = 0; k < VEC_STEPS; ++k) {
+    const int i = (threadIdx.x + NT * k) * 4;
+    if (i < width) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sm += keep[k][j];
+    }
+  }
+  const float mean = block_sum_sync<NW>(sm, scratch) * inv_w;
+  float sv = 0.f;
+#pragma unroll
+  for (int k = 0; k < VEC_STEPS; ++k) {
+    const int i = (threadIdx.x + NT * k) * 4;
+    if (i < width) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        keep[k][j] -= mean;
+        sv += keep[k][j] * keep[k][j];
+      }
+    }
+  }
+  sv = block_sum_sync<NW>(sv, scratch);
+  const float inv = 1.0f / sqrtf(sv * inv_w + eps);
+#pragma unroll
+  for (int k = 0; k < VEC_STEPS; ++k) {
+    const int i = (threadIdx.x + NT * k) * 4;
+    if (i < width) {
+      float w[4], o[4];
+      ld4<float>(next_weight + i, w);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = keep[k][j] * inv * w[j];
       st4<TO>(out + row * width + i, o);
     }
   }
@@ -417,6 +572,44 @@ extern "C" hipError_t ks_post_norm_add_rms_norm(
   } else {
     if (out_is_f32) launch_post_norm<short, float>(PN_ARGS);
     else launch_post_norm<short, short>(PN_ARGS);
+  }
+  HIP_CHECK_KERNEL();
+  return hipSuccess;
+}
+
+template <typename TD, typename TO>
+void launch_post_ln(bool vec, void* residual, const void* delta,
+                    long delta_stride, const void* weight, float mult,
+                    float eps, void* out, const void* next_weight, int rows,
+                    int width, hipStream_t stream) {
+  auto fn = vec ? post_layer_norm_add_vec4_kernel<TD, TO>
+                : post_layer_norm_add_kernel<TD, TO>;
+  hipLaunchKernelGGL(fn, dim3(rows), dim3(NT), 0, stream, (float*)residual,
+                     (const TD*)delta, delta_stride, (const float*)weight, mult,
+                     eps, (TO*)out, (const float*)next_weight, width);
+}
+
+extern "C" hipError_t ks_post_layer_norm_add(
+    void* residual, const void* delta, long delta_stride, int delta_is_f32,
+    const void* weight, float mult, float eps, void* out, int out_is_f32,
+    const void* next_weight, int rows, int width, hipStream_t stream) {
+  if (rows == 0) return hipSuccess;
+  if (delta && !weight) return hipErrorInvalidValue;
+  if (!delta && !out) return hipSuccess;
+  auto al = [](const void* p, int bytes) { return ((uintptr_t)p % bytes) == 0; };
+  const bool vec = width % 4 == 0 && width <= NT * 4 * VEC_STEPS &&
+                   delta_stride % 4 == 0 && al(residual, 16) && al(weight, 16) &&
+                   al(next_weight, 16) && al(delta, delta_is_f32 ? 16 : 8) &&
+                   al(out, out_is_f32 ? 16 : 8);
+#define PLN_ARGS                                                             \
+  vec, residual, delta, delta_stride, weight, mult, eps, out, next_weight,   \
+      rows, width, stream
+  if (delta_is_f32) {
+    if (out_is_f32) launch_post_ln<float, float>(PLN_ARGS);
+    else launch_post_ln<float, short>(PLN_ARGS);
+  } else {
+    if (out_is_f32) launch_post_ln<short, float>(PLN_ARGS);
+    else launch_post_ln<short, short>(PLN_ARGS);
   }
   HIP_CHECK_KERNEL();
   return hipSuccess;
