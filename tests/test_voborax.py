@@ -1,0 +1,606 @@
+"""The Voborax decoder through the engine, against the float64 oracle in
+voborax_oracle.py.
+
+Every test builds its own small config and random checkpoint. The same tests
+run on the CPU (plain torch forms of the ops, the engine's scheduling and page
+logic) and — marked gpu — on the HIP kernels in both activation dtypes.
+"""
+
+import json
+import os
+import sys
+
+import pytest
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+import voborax_oracle as O  # noqa: E402
+
+from kserve_amd.engine.config import (  # noqa: E402
+    CacheConfig,
+    EngineConfig,
+    HybridModelConfig,
+    MLPSpec,
+    SchedulerConfig,
+    SoftmaxMoESpec,
+)
+from kserve_amd.engine.engine import LLMEngine  # noqa: E402
+from kserve_amd.engine.replay import TraceReplayer  # noqa: E402
+from kserve_amd.engine.sampling_params import SamplingParams  # noqa: E402
+from kserve_amd.models.registry import build_model  # noqa: E402
+
+BACKENDS = [
+    pytest.param(("cpu", "float32"), id="cpu-f32"),
+    pytest.param(("cuda", "float32"), id="gpu-f32", marks=pytest.mark.gpu),
+    pytest.param(("cuda", "bfloat16"), id="gpu-bf16", marks=pytest.mark.gpu),
+]
+
+
+def varied_config(**kw):
+    """Six layers that differ in every size: windows of 5, 16 and 21, a layer
+    without feed-forward, two layers that read layer 0's rows (one of them
+    through another window and head count), experts with 0, 1 and 3 identity
+    outputs, with and without a shared expert, top 1 and 3."""
+    kw.setdefault("emb_scale", 0.7)
+    kw.setdefault("mult", 0.8)
+    return O.make_config(
+        layers=[
+            O.windowed(heads=4, dim=16, vdim=8, kv_rank=24, q_rank=20, rot_dim=8,
+                       rot_base=100.0, window=16, mlp=O.dense_cfg(40)),
+            O.windowed(heads=3, dim=8, vdim=12, kv_rank=24, q_rank=12, rot_dim=8,
+                       rot_base=100.0, window=5, kv_from=0,
+                       mlp=O.moe_cfg(experts=5, top=3, ff=10, identity=1, shared_ff=6)),
+            O.sinked(heads=2, dim=12, vdim=20, kv_rank=40, q_rank=28, mlp=None),
+            O.windowed(heads=6, dim=4, vdim=16, kv_rank=24, q_rank=16, rot_dim=8,
+                       rot_base=100.0, window=21, kv_from=0, mlp=O.dense_cfg(24)),
+            O.windowed(heads=1, dim=24, vdim=24, kv_rank=16, q_rank=32, rot_dim=12,
+                       rot_base=30.0, window=16,
+                       mlp=O.moe_cfg(experts=3, top=1, ff=16, identity=3)),
+            O.sinked(heads=5, dim=8, vdim=8, kv_rank=32, q_rank=8,
+                     mlp=O.moe_cfg(experts=4, top=2, ff=12, shared_ff=20)),
+        ],
+        **kw,
+    )
+
+
+def make_engine(cfg, sd, backend, num_blocks=64, block_size=16, max_seqs=4,
+                eager=False, multi_step=1, max_len=512, batched_tokens=None,
+                mixed=False):
+    device, dtype = backend
+    mc = HybridModelConfig.from_dict(cfg)
+    mc.dtype = dtype
+    model = build_model(mc, device=device)
+    model.load_hf_state_dict(sd)
+    ec = EngineConfig(
+        model=mc,
+        cache=CacheConfig(block_size=block_size, num_gpu_blocks=num_blocks),
+        scheduler=SchedulerConfig(
+            max_num_seqs=max_seqs,
+            max_num_batched_tokens=batched_tokens or max_len,
+            max_model_len=max_len, enable_chunked_prefill=True,
+            multi_step=multi_step, mixed_batches=mixed,
+        ),
+        device=device, eos_token_id=-1, enforce_eager=eager,
+    )
+    return LLMEngine(ec, model=model)
+
+
+def weights_for(cfg, backend, seed=0):
+    dt = torch.bfloat16 if backend[1] == "bfloat16" else torch.float32
+    return {k: v.float() for k, v in O.random_weights(cfg, seed=seed, dtype=dt).items()}
+
+
+def oracle(cfg, sd, toks):
+    return O.forward(cfg, {k: v.double() for k, v in sd.items()}, toks)[0]
+
+
+def rel_err(got, want):
+    """Centered RMS difference over the vocabulary, relative to the RMS of
+    the expected logits."""
+    got, want = got.double().cpu(), want.double()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    scale = (want - want.mean(-1, keepdim=True)).pow(2).mean().sqrt()
+    return (d.pow(2).mean(-1).sqrt() / scale).max().item()
+
+
+def tol(backend):
+    # bf16: worst position of a few hundred, inputs and products rounded
+    return 6e-2 if backend[1] == "bfloat16" else 2e-4
+
+
+def pos_errs(got, want):
+    return [rel_err(got[p : p + 1], want[p : p + 1]) for p in range(want.shape[0])]
+
+
+def agrees(got, want, backend, limit=None):
+    """fp32: every position within the tolerance. bf16 with routed experts:
+    the gap between the last chosen and the first rejected expert is now and
+    then smaller than what bf16 rounding does to the router's input; such a
+    token takes another expert than the float64 oracle (and moves the later
+    tokens that see it), which is no fault of the kernels. So nine positions
+    in ten must be within the tolerance and the median far inside it. Tests
+    without routed experts use the strict form in both dtypes."""
+    limit = limit or tol(backend)
+    if backend[1] == "float32":
+        return rel_err(got, want) < limit
+    errs = sorted(pos_errs(got, want))
+    n = len(errs)
+    return errs[(9 * n) // 10 - 1 if n >= 10 else 0] < limit and errs[n // 2] < limit / 2
+
+
+def run_schedule(engine, prompts, schedule):
+    """schedule: list of steps, each a list of (request index, count); every
+    token's logits are collected. Returns {index: [T, vocab]}."""
+    rp = TraceReplayer(engine)
+    at = {i: 0 for i in range(len(prompts))}
+    got = {i: [] for i in range(len(prompts))}
+    for step in schedule:
+        entries, end, order = [], [], []
+        for i, n in step:
+            lo = at[i]
+            entries.append(
+                {"id": f"r{i}", "tokens": prompts[i][lo : lo + n], "want": list(range(n))}
+            )
+            order.append((i, n))
+            at[i] = lo + n
+            if at[i] == len(prompts[i]):
+                end.append(f"r{i}")
+        logits = rp.step(entries, end)
+        off = 0
+        for i, n in order:
+            got[i].append(logits[off : off + n].float().cpu())
+            off += n
+    return {i: torch.cat(v) for i, v in got.items() if v}
+
+
+def random_prompt(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+@pytest.fixture(scope="module", params=BACKENDS)
+def backend(request):
+    if request.param[0] == "cuda":
+        from kserve_amd import ops
+
+        assert ops.has_native_seq(), "kserve_amd_seq_C must be built on a GPU box"
+    return request.param
+
+
+class TestWholePrompts:
+    def test_logits_and_residual_stream(self, backend):
+        cfg = varied_config()
+        sd = weights_for(cfg, backend)
+        eng = make_engine(cfg, sd, backend)
+        toks = random_prompt(75, cfg["vocab"], 1)
+        want, res = O.forward(cfg, {k: v.double() for k, v in sd.items()}, toks)
+        eng.model.debug_residuals = []
+        got = run_schedule(eng, [toks], [[(0, len(toks))]])[0]
+        streams = eng.model.debug_residuals
+        eng.model.debug_residuals = None
+        assert len(streams) == len(cfg["layers"]) == len(res)
+        ok = 0
+        for mine, ref in zip(streams, res):
+            scale = ref.abs().max().item()
+            err = (mine.double().cpu() - ref).abs().amax(-1) / scale
+            ok += int((err < tol(backend) * 4).float().mean().item() >= 0.9)
+        assert ok == len(res)
+        assert agrees(got, want, backend)
+
+    def test_first_tokens(self, backend):
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=3)
+        eng = make_engine(cfg, sd, backend)
+        for n in (1, 2, 3):
+            toks = random_prompt(n, cfg["vocab"], 10 + n)
+            got = run_schedule(eng, [toks], [[(0, n)]])[0]
+            assert agrees(got, oracle(cfg, sd, toks), backend)
+
+    def test_sizes_of_one_and_odd_sizes(self, backend):
+        """One head, a window of one position (a token sees itself only),
+        one expert, every router output an identity, odd sizes everywhere."""
+        cfg = O.make_config(
+            vocab=31, width=18, emb_scale=1.0, mult=1.0, eps=1e-6,
+            layers=[
+                O.windowed(heads=1, dim=6, vdim=22, kv_rank=10, q_rank=6, rot_dim=2,
+                           window=1, mlp=O.moe_cfg(experts=1, top=1, ff=8)),
+                O.sinked(heads=3, dim=4, vdim=2, kv_rank=6, q_rank=10,
+                         mlp=O.moe_cfg(experts=2, top=4, ff=6, identity=2, shared_ff=2)),
+                O.windowed(heads=2, dim=10, vdim=6, kv_rank=10, q_rank=14, rot_dim=2,
+                           window=3, kv_from=0, mlp=O.dense_cfg(7)),
+            ],
+        )
+        sd = weights_for(cfg, backend, seed=4)
+        eng = make_engine(cfg, sd, backend)
+        toks = random_prompt(21, cfg["vocab"], 5)
+        got = run_schedule(eng, [toks], [[(0, 12)]] + [[(0, 1)]] * 9)[0]
+        assert agrees(got, oracle(cfg, sd, toks), backend)
+
+    def test_many_experts_take_the_sorted_path(self, backend):
+        """More tokens than the small-batch expert path takes, more router
+        outputs than a wave has lanes; some experts get no token at all."""
+        cfg = O.make_config(
+            vocab=40, width=32,
+            layers=[O.sinked(heads=2, dim=8, vdim=8,
+                             mlp=O.moe_cfg(experts=66, top=2, ff=8, identity=4,
+                                           shared_ff=8))],
+        )
+        sd = weights_for(cfg, backend, seed=19)
+        eng = make_engine(cfg, sd, backend)
+        toks = random_prompt(50, cfg["vocab"], 20)
+        got = run_schedule(eng, [toks], [[(0, 50)]])[0]
+        want = oracle(cfg, sd, toks)
+        if backend[1] == "float32":
+            assert rel_err(got, want) < tol(backend)
+        else:
+            assert sum(e < tol(backend) for e in pos_errs(got, want)) >= 40
+
+
+class TestSchedules:
+    def test_prefill_then_decode(self, backend):
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=5)
+        eng = make_engine(cfg, sd, backend)
+        toks = random_prompt(70, cfg["vocab"], 6)
+        want = oracle(cfg, sd, toks)
+        sched = [[(0, 30)]] + [[(0, 1)] for _ in range(40)]
+        got = run_schedule(eng, [toks], sched)[0]
+        assert agrees(got, want, backend)
+
+    def test_decode_graphs_equal_eager(self, backend):
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=21)
+        toks = random_prompt(50, cfg["vocab"], 22)
+        sched = [[(0, 9)]] + [[(0, 1)] for _ in range(41)]
+        a = run_schedule(make_engine(cfg, sd, backend), [toks], sched)[0]
+        b = run_schedule(make_engine(cfg, sd, backend, eager=True), [toks], sched)[0]
+        assert agrees(a, b.double(), backend, tol(backend) / 4)
+
+    def test_token_by_token_from_the_start(self, backend):
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=6)
+        eng = make_engine(cfg, sd, backend)
+        toks = random_prompt(45, cfg["vocab"], 7)
+        got = run_schedule(eng, [toks], [[(0, 1)] for _ in toks])[0]
+        assert agrees(got, oracle(cfg, sd, toks), backend)
+
+    @pytest.mark.parametrize("sizes", [[2] * 25, [3, 17, 2, 16, 1, 5, 2, 2, 31],
+                                       [16, 16, 16, 1, 15, 2, 14], [7, 8, 1, 1, 20, 33]])
+    def test_portions(self, backend, sizes):
+        """Portions down to two tokens, cut inside pages and inside windows
+        and exactly at their ends."""
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=7)
+        eng = make_engine(cfg, sd, backend)
+        toks = random_prompt(sum(sizes), cfg["vocab"], 8)
+        got = run_schedule(eng, [toks], [[(0, n)] for n in sizes])[0]
+        assert agrees(got, oracle(cfg, sd, toks), backend)
+
+    def test_mixed_batches_and_reuse(self, backend):
+        """Unequal requests side by side — portions next to decode tokens,
+        requests skipped for a step — in a pool too small for all of them at
+        once, so pages are handed out again (with what they held before)."""
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=8)
+        # 9 usable pages of 16; six requests
+        eng = make_engine(cfg, sd, backend, num_blocks=10, max_seqs=3)
+        lens = [40, 23, 9, 33, 17, 48]
+        prompts = [random_prompt(n, cfg["vocab"], 20 + i) for i, n in enumerate(lens)]
+        sched = [
+            [(0, 19), (1, 5)],
+            [(0, 1), (1, 16), (2, 2)],
+            [(0, 1), (2, 1)],
+            [(1, 1), (2, 1), (0, 19)],      # request 0 done
+            [(1, 1), (2, 5)],               # requests 1, 2 done
+            [(3, 33), (4, 3)],              # request 3 done
+            [(4, 1), (5, 20)],
+            [(4, 1)],
+            [(5, 1), (4, 12)],              # request 4 done
+        ] + [[(5, 1)] for _ in range(27)]
+        got = run_schedule(eng, prompts, sched)
+        for i, toks in enumerate(prompts):
+            assert got[i].shape[0] == len(toks)
+            assert agrees(got[i], oracle(cfg, sd, toks), backend), i
+        assert eng.scheduler.block_manager.num_free_blocks == 9
+        assert eng.scheduler.state_slots is None   # nothing recurrent to keep
+
+    def test_alone_equals_batched(self, backend):
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=9)
+        prompts = [random_prompt(n, cfg["vocab"], 40 + n) for n in (26, 7, 18)]
+        eng = make_engine(cfg, sd, backend)
+        together = run_schedule(
+            eng, prompts,
+            [[(0, 20), (1, 7), (2, 3)], [(0, 1), (2, 15)]] + [[(0, 1)]] * 5,
+        )
+        for i, toks in enumerate(prompts):
+            alone = run_schedule(eng, [toks], [[(0, len(toks))]])[0]
+            # same kernels, other batch composition: rounding only
+            assert agrees(together[i], alone.double(), backend, tol(backend) / 4)
+
+    def test_long_decode(self, backend):
+        cfg = O.make_config(
+            vocab=50, width=32,
+            layers=[
+                O.windowed(heads=2, dim=8, vdim=16, kv_rank=16, q_rank=16,
+                           rot_dim=8, window=70, mlp=O.moe_cfg(experts=3, top=2, ff=8)),
+                O.sinked(heads=2, dim=8, vdim=8, mlp=None),
+            ],
+        )
+        sd = weights_for(cfg, backend, seed=10)
+        eng = make_engine(cfg, sd, backend, num_blocks=32)
+        toks = random_prompt(300, cfg["vocab"], 11)
+        got = run_schedule(eng, [toks], [[(0, 4)]] + [[(0, 1)]] * 296)[0]
+        assert agrees(got, oracle(cfg, sd, toks), backend)
+
+
+class TestNeedles:
+    """One mixer whose weights make a single key decide the output of every
+    query that can see it: a key lost at a page border, cut off by a tile,
+    or a window that is one position off shows at once."""
+
+    D = 8
+
+    def _setup(self, backend, window, needle, total, second_reader=False):
+        kind = O.windowed if window else O.sinked
+        kw = dict(heads=2, dim=self.D, vdim=8, kv_rank=12, q_rank=10, scale=1.0,
+                  mlp=None)
+        if window:
+            kw.update(rot_dim=4, rot_base=100.0, window=window)
+        layers = [kind(**kw)]
+        if second_reader:
+            # a second layer reads the first one's rows through its own window
+            kw2 = dict(kw, kv_from=0, window=window + 3, heads=3)
+            layers.append(O.windowed(**kw2))
+        cfg = O.make_config(vocab=40, width=16, emb_scale=1.0, layers=layers)
+        sd = weights_for(cfg, backend, seed=12)
+        W = cfg["width"]
+        # Every embedding = a common direction (coordinate 0) plus noise in
+        # the coordinates from 2 on; token 1 (the needle) also has
+        # coordinate 1.
+        g = torch.Generator().manual_seed(77)
+        emb = torch.randn(cfg["vocab"], W, generator=g) * 0.5
+        emb[:, 0] = 1.0
+        emb[:, 1] = 0.0
+        emb[1, 1] = 3.0
+        sd["embed"] = emb
+        for i in range(len(layers)):
+            p = f"l{i}.mix."
+            H = layers[i]["mixer"]["heads"]
+            rd = layers[i]["mixer"].get("rot_dim", 0)
+            # query latent 0 reads the common direction; the last unrotated
+            # coordinate of every head reads that latent, nothing else does
+            sd[p + "dq"].zero_()
+            sd[p + "dq"][0, 0] = 1.0
+            sd[p + "dq.norm"].fill_(1.0)
+            sd[p + "uq"].zero_()
+            for h in range(H):
+                sd[p + "uq"][h * (self.D + rd) + self.D - 1, 0] = 1.5
+            # kv latent 0 reads the needle coordinate, latent 1 the common
+            # one; each head's last key coordinate reads latent 0, so every
+            # other key is zero and the needle's score stands far above
+            if i == 0:
+                sd[p + "dkv"].zero_()
+                sd[p + "dkv"][0, 1] = 1.0
+                sd[p + "dkv"][1, 0] = 1.0
+                sd[p + "dkv.norm"].fill_(1.0)
+            sd[p + "uk"].zero_()
+            for h in range(H):
+                sd[p + "uk"][h * self.D + self.D - 1, 0] = 1.0
+            if (p + "sink") in sd:
+                sd[p + "sink"].fill_(-2.0)
+        dt = torch.bfloat16 if backend[1] == "bfloat16" else torch.float32
+        sd = {k: v.to(dt).float() for k, v in sd.items()}
+        toks = [2 + (i % 30) for i in range(total)]
+        toks[needle] = 1
+        return cfg, sd, toks
+
+    def _check_power(self, cfg, sd, toks, needle, want, inside, outside):
+        plain = list(toks)
+        plain[needle] = 3
+        other = oracle(cfg, sd, plain)
+        for p in inside:     # the needle matters where it is visible
+            assert rel_err(other[p : p + 1], want[p : p + 1]) > 0.1, p
+        for p in outside:    # and not at all where it is not
+            assert rel_err(other[p : p + 1], want[p : p + 1]) < 1e-9, p
+
+    @pytest.mark.parametrize("needle", [0, 15, 16, 63, 64, 65, 127, 128])
+    def test_far_key_at_page_borders(self, backend, needle):
+        """No window: the key stays visible from hundreds of positions away,
+        in the prompt and while decoding."""
+        cfg, sd, toks = self._setup(backend, 0, needle, 330)
+        want = oracle(cfg, sd, toks)
+        self._check_power(cfg, sd, toks, needle, want, [needle, 200, 329], [])
+        eng = make_engine(cfg, sd, backend, num_blocks=32)
+        got = run_schedule(eng, [toks], [[(0, 270)]] + [[(0, 1)]] * 60)[0]
+        assert rel_err(got, want) < tol(backend)
+
+    @pytest.mark.parametrize("window", [16, 24, 64, 50, 2])
+    def test_window_edges_in_prompt_and_decode(self, backend, window):
+        """The query window-1 positions after the needle is the last one that
+        sees it. Queries around that edge are run inside a prompt portion,
+        decoded one by one, and in portions cut right at the edge."""
+        needle = 2 * window + 3
+        edge = needle + window - 1
+        T = edge + 12
+        cfg, sd, toks = self._setup(backend, window, needle, T)
+        want = oracle(cfg, sd, toks)
+        self._check_power(cfg, sd, toks, needle, want, [needle, edge],
+                          [needle - 1, edge + 1, edge + 2, T - 1])
+        eng = make_engine(cfg, sd, backend, num_blocks=32)
+        scheds = [
+            [[(0, T)]],
+            [[(0, needle + 1)]] + [[(0, 1)]] * (T - needle - 1),
+            [[(0, edge)], [(0, 1)], [(0, 2)], [(0, T - edge - 3)]],
+            [[(0, edge + 1)], [(0, T - edge - 1)]],
+            [[(0, edge - 1)], [(0, 2)], [(0, 2)], [(0, T - edge - 3)]],
+        ]
+        for sched in scheds:
+            got = run_schedule(eng, [toks], sched)[0]
+            assert rel_err(got, want) < tol(backend), sched[:2]
+
+    def test_a_second_layer_reads_the_same_rows(self, backend):
+        """Layer 1 has no kv projection and a window three positions longer
+        than layer 0's: the needle row written by layer 0 serves both."""
+        window = 20
+        needle = 45
+        T = needle + window + 15
+        cfg, sd, toks = self._setup(backend, window, needle, T, second_reader=True)
+        want = oracle(cfg, sd, toks)
+        self._check_power(cfg, sd, toks, needle, want,
+                          [needle, needle + window - 1, needle + window + 2],
+                          [needle - 1, needle + window + 3, T - 1])
+        eng = make_engine(cfg, sd, backend, num_blocks=32)
+        for sched in ([[(0, T)]],
+                      [[(0, needle + window)]] + [[(0, 1)]] * (T - needle - window),
+                      [[(0, 31)], [(0, 33)], [(0, 2)], [(0, T - 66)]]):
+            got = run_schedule(eng, [toks], sched)[0]
+            assert rel_err(got, want) < tol(backend), sched[:2]
+
+
+class TestGeneration:
+    def test_greedy_through_scheduler(self, backend):
+        """LLMEngine.generate: the scheduler's own prefill/decode batching,
+        sampling, multi-step decode windows."""
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=13)
+        eng = make_engine(cfg, sd, backend, multi_step=4)
+        prompts = [random_prompt(n, cfg["vocab"], 60 + n) for n in (5, 19, 11)]
+        outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12,
+                                                     ignore_eos=True))
+        assert len(outs) == 3
+        for p, o in zip(prompts, outs.values()):
+            assert len(o.output_token_ids) == 12
+            if backend[1] == "bfloat16":
+                continue  # near-ties may flip; the logits are checked above
+            seq = list(p)
+            for t in o.output_token_ids:
+                logits = oracle(cfg, sd, seq)[-1]
+                top2 = logits.topk(2).values
+                if (top2[0] - top2[1]).item() > 1e-3:
+                    assert int(logits.argmax()) == t
+                seq.append(t)
+
+    def test_mixed_batches_in_the_scheduler(self, backend):
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=18)
+        prompts = [random_prompt(n, cfg["vocab"], 90 + n) for n in (20, 18, 21)]
+        sp = SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True)
+        plain = make_engine(cfg, sd, backend, batched_tokens=24).generate(prompts, sp)
+        mixed = make_engine(cfg, sd, backend, batched_tokens=24, mixed=True).generate(
+            prompts, sp
+        )
+        if backend[1] == "float32":
+            for a, b in zip(plain.values(), mixed.values()):
+                assert a.output_token_ids == b.output_token_ids
+
+    def test_preemption_in_a_tight_pool(self, backend):
+        cfg = varied_config()
+        sd = weights_for(cfg, backend, seed=14)
+        prompts = [random_prompt(n, cfg["vocab"], 80 + n) for n in (30, 28, 25)]
+        sp = SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)
+        roomy = make_engine(cfg, sd, backend, num_blocks=64).generate(prompts, sp)
+        tight = make_engine(cfg, sd, backend, num_blocks=8, max_seqs=3).generate(prompts, sp)
+        if backend[1] == "float32":
+            for a, b in zip(roomy.values(), tight.values()):
+                assert a.output_token_ids == b.output_token_ids
+
+
+class TestConfigAndRegistry:
+    def test_config_json_roundtrip(self, tmp_path):
+        from kserve_amd.models.registry import load_model_config, native_modules_for
+
+        cfg = varied_config()
+        (tmp_path / "config.json").write_text(json.dumps(cfg))
+        mc = load_model_config(str(tmp_path))
+        assert isinstance(mc, HybridModelConfig) and mc.architecture == "Voborax"
+        assert (mc.residual_mult, mc.embedding_scale) == (0.8, 0.7)
+        lt = [l.latent for l in mc.layers]
+        assert [x.window for x in lt] == [16, 5, 0, 21, 16, 0]
+        assert [x.kv_from for x in lt] == [None, 0, None, 0, None, None]
+        assert [(x.gate, x.sink) for x in lt[:3]] == [(True, False)] * 2 + [(False, True)]
+        assert (lt[4].rot_dim, lt[4].rot_dims, lt[4].rot_base) == (12, 12, 30.0)
+        assert lt[2].rot_dim == 0 and lt[2].cache_dim == 40 and lt[0].cache_dim == 32
+        m = mc.layers[1].mlp
+        assert isinstance(m, SoftmaxMoESpec)
+        assert (m.experts, m.identity, m.top, m.ff, m.shared_ff) == (5, 1, 3, 10, 6)
+        assert isinstance(mc.layers[0].mlp, MLPSpec) and mc.layers[0].mlp.ff == 40
+        assert mc.layers[2].mlp is None and mc.layers[4].mlp.shared_ff == 0
+        assert native_modules_for(str(tmp_path)) == ("kserve_amd_seq_C",)
+
+    def test_pages_only_where_rows_are_written(self):
+        mc = HybridModelConfig.from_dict(varied_config())
+        model = build_model(mc, device="cpu")
+        layout = model.cache_layout()
+        assert [kv for kv, _ in layout] == [
+            (1, 32, 0), None, (1, 40, 0), None, (1, 28, 0), (1, 32, 0)
+        ]
+        assert all(state == {} for _, state in layout)
+        assert mc.kv_bytes_per_block(16, 2) == (32 + 40 + 28 + 32) * 16 * 2
+
+    def test_kv_from_must_point_at_a_writer(self):
+        cfg = varied_config()
+        cfg["layers"][3]["mixer"]["kv_from"] = 1     # layer 1 reads layer 0 itself
+        with pytest.raises(ValueError):
+            build_model(HybridModelConfig.from_dict(cfg), device="cpu")
+
+    def test_server_cli_picks_the_engine(self, tmp_path):
+        from kserve_amd.runtimes.huggingfaceserver import detect_backend
+
+        (tmp_path / "config.json").write_text(json.dumps(varied_config()))
+        assert detect_backend(str(tmp_path)) == "engine"
+
+    def test_checkpoint_loading_from_safetensors(self, tmp_path):
+        from safetensors.torch import save_file
+
+        from kserve_amd.engine.weights import load_safetensors_weights
+
+        cfg = varied_config()
+        sd = O.random_weights(cfg, seed=15, dtype=torch.bfloat16)
+        save_file({k: v.to(torch.bfloat16).contiguous() for k, v in sd.items()},
+                  str(tmp_path / "model.safetensors"))
+        mc = HybridModelConfig.from_dict(cfg)
+        mc.dtype = "float32"
+        model = build_model(mc, device="cpu")
+        load_safetensors_weights(model, str(tmp_path))
+        a = model.layers[0].attn
+        assert torch.equal(a.in_proj[:20], sd["l0.mix.dq"].float())
+        assert torch.equal(a.in_proj[20:52], sd["l0.mix.dkv"].float())
+        assert torch.equal(a.in_proj[52:], sd["l0.mix.g"].float())
+        assert torch.equal(a.uk[2], sd["l0.mix.uk"].float()[32:48])
+        assert torch.equal(a.uv_t[1], sd["l0.mix.uv"].float()[8:16].T)
+        assert torch.equal(model.layers[2].attn.sink, sd["l2.mix.sink"].float())
+        m = model.layers[1].mlp
+        assert torch.equal(m.gate_up[4, 10:], sd["l1.mlp.e4.up"].float())
+        assert torch.equal(m.down[:, 3], sd["l1.mlp.e3.down"].float())
+        assert torch.equal(m.correction, sd["l1.mlp.correction"].float())
+        assert m.router.shape == (6, 32)
+
+
+class TestExpertsAtScale:
+    """The routed feed-forward alone on thousands of tokens (sorted form)
+    and on a decode-sized batch (all-experts form), against the oracle."""
+
+    @pytest.mark.parametrize("tokens", [200, 3000])
+    def test_both_forms(self, backend, tokens):
+        from kserve_amd.models.mixers import SoftmaxRoutedMoE
+
+        W = 256
+        f = O.moe_cfg(experts=8, top=2, ff=512, identity=2, shared_ff=128)
+        cfg = O.make_config(width=W, layers=[O.sinked(mlp=f)])
+        sd = weights_for(cfg, backend, seed=30)
+        dt = torch.bfloat16 if backend[1] == "bfloat16" else torch.float32
+        mod = SoftmaxRoutedMoE(W, SoftmaxMoESpec.from_dict(f), dt).to(backend[0])
+        mod.load(lambda n: sd[n], "l0.mlp.")
+        assert (tokens <= mod.dense_max_tokens) == (tokens == 200)
+        g = torch.Generator().manual_seed(31)
+        h = torch.randn(tokens, W, generator=g).to(dt).float()
+        got = mod(h.to(dt).to(backend[0]))
+        assert got.dtype == torch.float32
+        want = O.moe_ff(h.double(), {k: v.double() for k, v in sd.items()}, "l0.mlp.", f)
+        err = (got.double().cpu() - want).pow(2).mean(-1).sqrt() / want.pow(2).mean().sqrt()
+        limit = 3e-2 if backend[1] == "bfloat16" else 1e-4
+        # bf16: a token whose second and third scores are closer than the
+        # rounding of the router's input may take another expert
+        assert (err < limit).float().mean().item() >= (0.97 if dt == torch.bfloat16 else 1.0)

@@ -176,3 +176,111 @@ def forward(cfg, w, tokens):
         stream.append(x.clone())
     y = layer_norm(x, w["final.norm"], eps)
     return y @ w["head"].T, stream
+
+
+# -- small configurations and random checkpoints for the tests ----------------
+
+def mixer(heads=2, dim=8, vdim=8, kv_rank=16, q_rank=16, scale=None, rot_dim=0,
+          rot_base=10000.0, window=0, kv_from=None):
+    m = {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": kv_rank,
+         "q_rank": q_rank, "scale": scale if scale is not None else (dim + rot_dim) ** -0.5}
+    if rot_dim:
+        m["rot_dim"] = rot_dim
+        m["rot"] = {"base": rot_base, "dims": rot_dim}
+    if window:
+        m["mask"] = {"size": window}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return m
+
+
+def dense_cfg(ff=32):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe_cfg(experts=4, top=2, ff=16, identity=0, shared_ff=0):
+    d = {"kind": "moe", "expert": {"ff": ff},
+         "router": {"experts": experts, "identity": identity, "top": top}}
+    if shared_ff:
+        d["shared"] = {"ff": shared_ff}
+    return d
+
+
+def windowed(mlp="dense", **kw):
+    """A layer with rotated key part, sliding window and output gate."""
+    kw.setdefault("rot_dim", 8)
+    kw.setdefault("window", 16)
+    return {"type": "latent_attention", "mixer": mixer(**kw),
+            "mlp": dense_cfg() if mlp == "dense" else mlp}
+
+
+def sinked(mlp="dense", **kw):
+    """A layer without positions: causal, with a sink."""
+    return {"type": "latent_attention_2", "mixer": mixer(**kw),
+            "mlp": dense_cfg() if mlp == "dense" else mlp}
+
+
+def make_config(layers, vocab=48, width=32, eps=1e-5, emb_scale=1.0, mult=1.0):
+    return {"architecture": "Voborax", "vocab": vocab, "width": width,
+            "embedding": {"scale": emb_scale}, "norm": {"eps": eps},
+            "residual_mult": mult, "layers": layers}
+
+
+def random_weights(cfg, seed=0, dtype=torch.float32):
+    """name -> tensor, values rounded to ``dtype`` and returned as float64."""
+    g = torch.Generator().manual_seed(seed)
+    W = int(cfg["width"])
+    out = {}
+
+    def mat(name, rows, cols, gain=1.0):
+        out[name] = torch.randn(rows, cols, generator=g) * gain * cols ** -0.5
+
+    def vec(name, n, mean=0.0, std=0.3):
+        out[name] = mean + torch.randn(n, generator=g) * std
+
+    out["embed"] = torch.randn(int(cfg["vocab"]), W, generator=g)
+    mat("head", int(cfg["vocab"]), W)
+    vec("final.norm", W, 1.0)
+    for i, L in enumerate(cfg["layers"]):
+        p, mx = f"l{i}.", L["mixer"]
+        H, D, DV = mx["heads"], mx["dim"], mx["vdim"]
+        R, Q, rd = mx["kv_rank"], mx["q_rank"], mx.get("rot_dim", 0)
+        vec(p + "norm1", W, 1.0)
+        mat(p + "mix.dq", Q, W)
+        vec(p + "mix.dq.norm", Q, 1.0)
+        mat(p + "mix.uq", H * (D + rd), Q, 2.0)
+        if mx.get("kv_from") is None:
+            mat(p + "mix.dkv", R + rd, W)
+            vec(p + "mix.dkv.norm", R, 1.0)
+        mat(p + "mix.uk", H * D, R, 2.0)
+        mat(p + "mix.uv", H * DV, R)
+        mat(p + "mix.o", W, H * DV)
+        if L["type"] == "latent_attention":
+            mat(p + "mix.g", H, W, 2.0)
+        else:
+            vec(p + "mix.sink", H, 0.0, 1.0)
+        ml = L.get("mlp")
+        if not ml:
+            continue
+        vec(p + "norm2", W, 1.0)
+        q = p + "mlp."
+        if ml["kind"] == "dense":
+            mat(q + "up", ml["ff"], W)
+            vec(q + "up.b", ml["ff"])
+            mat(q + "down", W, ml["ff"])
+            vec(q + "down.b", W)
+            continue
+        r = ml["router"]
+        n_out = r["experts"] + r.get("identity", 0)
+        mat(q + "router", n_out, W, 3.0)
+        vec(q + "correction", n_out, 0.0, 0.1)
+        names = [f"e{e}." for e in range(r["experts"])]
+        ffs = [ml["expert"]["ff"]] * r["experts"]
+        if ml.get("shared"):
+            names.append("shared.")
+            ffs.append(ml["shared"]["ff"])
+        for n, ff in zip(names, ffs):
+            mat(q + n + "gate", ff, W)
+            mat(q + n + "up", ff, W)
+            mat(q + n + "down", W, ff)
+    return {k: v.to(dtype).to(F64) for k, v in out.items()}
