@@ -126,6 +126,60 @@ def _desalix_model_configs(size: dict, runs: int):
     return desalix, llama
 
 
+# layer shapes for --voborax-compare: the widths, head counts and experts of
+# DESALIX_SIZES; 128 unrotated + 64 rotated query/key coordinates per head,
+# a cached row of 192 latent + 64 rotated columns per token and layer
+VOBORAX_SIZES = {
+    "2k": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=192,
+               q_rank=768, window=1024, ff=4096, experts=8, top=2, vocab=32000),
+    "4k": dict(width=4096, heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=192,
+               q_rank=1536, window=1024, ff=7168, experts=8, top=2, vocab=32000),
+}
+
+
+def _voborax_model_configs(size: dict):
+    """A four-layer Voborax model (windowed + experts, windowed reading layer
+    0's rows + experts, windowed + dense, causal with sink + experts) and the
+    Desalix model of equal width, heads, depth and experts that
+    --desalix-compare measures."""
+    from kserve_amd.engine.config import (
+        HybridLayerSpec,
+        HybridModelConfig,
+        LatentAttentionSpec,
+        MLPSpec,
+        SoftmaxMoESpec,
+    )
+
+    def latent(window, sink, kv_from=None):
+        rot = 0 if sink else size["rot_dim"]
+        return LatentAttentionSpec(
+            heads=size["heads"], dim=size["dim"], vdim=size["vdim"],
+            kv_rank=size["kv_rank"] + (size["rot_dim"] - rot),
+            q_rank=size["q_rank"], scale=(size["dim"] + rot) ** -0.5,
+            rot_dim=rot, rot_dims=rot, rot_base=500000.0, window=window,
+            sink=sink, gate=not sink, kv_from=kv_from,
+        )
+
+    moe = SoftmaxMoESpec(experts=size["experts"], top=size["top"], ff=size["ff"],
+                         identity=1, shared_ff=0)
+    # two matrices instead of an expert's three: equal arithmetic per token
+    dense = MLPSpec(ff=3 * size["top"] * size["ff"] // 2)
+    w = size["window"]
+    voborax = HybridModelConfig(
+        vocab_size=size["vocab"], hidden_size=size["width"],
+        layers=[
+            HybridLayerSpec("latent_attention", latent=latent(w, False), mlp=moe),
+            HybridLayerSpec("latent_attention", latent=latent(w, False, 0), mlp=moe),
+            HybridLayerSpec("latent_attention", latent=latent(w, False), mlp=dense),
+            HybridLayerSpec("latent_attention_2", latent=latent(0, True), mlp=moe),
+        ],
+        model_name="voborax-bench", architecture="Voborax", residual_mult=0.7,
+    )
+    dsize = dict(DESALIX_SIZES["2k" if size["width"] == 2048 else "4k"])
+    desalix, _ = _desalix_model_configs(dsize, runs=4)
+    return voborax, desalix
+
+
 def _throughput(mcfg, prompt_len, n_prompts, concurrency, steps, warmup, eager):
     """(prefill tok/s, decode tok/s) through the engine's own step()."""
     import torch
@@ -271,6 +325,58 @@ def desalix_compare(args):
     return 0
 
 
+def voborax_compare(args):
+    """Prefill and decode tok/s of the Voborax design next to the Desalix
+    model of equal width, heads, depth and experts (the closest design the
+    engine serves: the same fp32 attention kernel and routed experts), both
+    through LLMEngine.step() on one GPU, bf16, random weights. One JSON line
+    per (size, model), each measured in a process of its own."""
+    import subprocess
+    import sys
+
+    if args.compare_only is None or "," in args.voborax_compare:
+        rc = 0
+        for name in args.voborax_compare.split(","):
+            for label in ("voborax", "desalix"):
+                if args.compare_only and args.compare_only != label:
+                    continue
+                cmd = [sys.executable, "-u", os.path.abspath(__file__),
+                       "--voborax-compare", name, "--compare-only", label,
+                       "--steps", str(args.steps), "--warmup", str(args.warmup),
+                       "--concurrency", str(args.concurrency),
+                       "--prompt-len", str(args.prompt_len)]
+                if args.eager:
+                    cmd.append("--eager")
+                rc = subprocess.call(cmd)
+                if rc != 0:
+                    return rc
+        return rc
+
+    import torch
+
+    assert torch.cuda.is_available(), "--voborax-compare needs a GPU"
+    name, label = args.voborax_compare, args.compare_only
+    size = VOBORAX_SIZES[name]
+    voborax, desalix = _voborax_model_configs(size)
+    mcfg = voborax if label == "voborax" else desalix
+    prefill, decode = _throughput(
+        mcfg, prompt_len=args.prompt_len if args.prompt_len != 512 else 2048,
+        n_prompts=8, concurrency=min(args.concurrency, 256),
+        steps=args.steps, warmup=args.warmup, eager=args.eager,
+    )
+    print(json.dumps({
+        "bench": "voborax-compare", "size": name, "model": mcfg.model_name,
+        "layers": 4, "width": size["width"],
+        "experts": size["experts"], "top": size["top"],
+        "prefill_tok_s": round(prefill, 1),
+        "decode_tok_s": round(decode, 1),
+        "prefill_batch": "8 x prompt", "decode_concurrency":
+            min(args.concurrency, 256),
+        "dtype": "bfloat16", "data": "synthetic, random-init weights",
+    }), flush=True)
+    return 0
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -316,10 +422,17 @@ def main():
                              "beside a llama model of equal width, heads, "
                              "depth and arithmetic per token (sizes: "
                              + ", ".join(DESALIX_SIZES) + ")")
+    parser.add_argument("--voborax-compare", type=str, default=None,
+                        metavar="SIZE[,SIZE...]",
+                        help="instead of the flagship workload: prefill and "
+                             "decode throughput of a Voborax-design model "
+                             "beside the Desalix model of equal width, heads, "
+                             "depth and experts (sizes: "
+                             + ", ".join(VOBORAX_SIZES) + ")")
     parser.add_argument("--compare-only", type=str, default=None,
-                        choices=["desalix", "llama"],
-                        help="with --desalix-compare: run one side only "
-                             "(e.g. under a profiler)")
+                        choices=["desalix", "llama", "voborax"],
+                        help="with --desalix-compare / --voborax-compare: run "
+                             "one side only (e.g. under a profiler)")
     parser.add_argument("--profile-cpu", action="store_true",
                         help="cProfile the timed loop and print hot functions")
     args = parser.parse_args()
@@ -327,6 +440,8 @@ def main():
         return hybrid_compare(args)
     if args.desalix_compare:
         return desalix_compare(args)
+    if args.voborax_compare:
+        return voborax_compare(args)
 
     import torch
 

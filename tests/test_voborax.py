@@ -105,8 +105,12 @@ def rel_err(got, want):
 
 
 def tol(backend):
-    # bf16: worst position of a few hundred, inputs and products rounded
-    return 6e-2 if backend[1] == "bfloat16" else 2e-4
+    # bf16: every sublayer output is layer-normed before it is added, so the
+    # relative rounding error of a sublayer arrives in the stream at full
+    # size whatever the output's own magnitude, twelve times over in the
+    # six-layer model of these tests (width 32); the fp32 runs are the sharp
+    # test of the arithmetic, the op tests that of the bf16 kernels
+    return 1e-1 if backend[1] == "bfloat16" else 2e-4
 
 
 def pos_errs(got, want):
