@@ -428,9 +428,10 @@ class LatentAttention(nn.Module):
             _param(s.kv_rank, dtype=torch.float32) if self.own_kv else None
         )
         self.uq = _param(s.heads * (s.dim + s.rot_dim), s.q_rank, dtype=dtype)
-        self.uk = _param(s.heads, s.dim, s.kv_rank, dtype=dtype)
-        # U_v stored transposed per head: [heads, kv_rank, vdim]
-        self.uv_t = _param(s.heads, s.kv_rank, s.vdim, dtype=dtype)
+        # U_k transposed per head, [heads, kv_rank, dim]: it maps a query
+        # head into latent coordinates; U_v as stored, [heads, vdim, kv_rank]
+        self.uk_t = _param(s.heads, s.kv_rank, s.dim, dtype=dtype)
+        self.uv = _param(s.heads, s.vdim, s.kv_rank, dtype=dtype)
         self.sink = _param(s.heads, dtype=torch.float32) if s.sink else None
         self.o_proj = _param(width, s.heads * s.vdim, dtype=dtype)
         self.register_buffer(
@@ -450,10 +451,10 @@ class LatentAttention(nn.Module):
         self.in_proj.copy_(torch.cat(parts, dim=0))
         self.q_norm.copy_(get(prefix + "dq.norm").float())
         self.uq.copy_(get(prefix + "uq").to(dt))
-        self.uk.copy_(get(prefix + "uk").to(dt).view(s.heads, s.dim, s.kv_rank))
-        self.uv_t.copy_(
-            get(prefix + "uv").to(dt).view(s.heads, s.vdim, s.kv_rank).transpose(1, 2)
+        self.uk_t.copy_(
+            get(prefix + "uk").to(dt).view(s.heads, s.dim, s.kv_rank).transpose(1, 2)
         )
+        self.uv.copy_(get(prefix + "uv").to(dt).view(s.heads, s.vdim, s.kv_rank))
         if self.sink is not None:
             self.sink.copy_(get(prefix + "sink").float())
         self.o_proj.copy_(get(prefix + "o").to(dt))
@@ -470,7 +471,7 @@ class LatentAttention(nn.Module):
         )
         q = F.linear(cq, self.uq)
         qf = ops.head_matmul_rope(
-            q, self.uk, s.heads, s.rot_dim, positions, self.inv_freq,
+            q, self.uk_t, s.heads, s.rot_dim, positions, self.inv_freq,
             torch.float32,
         )
         gate = proj[:, s.q_rank + self.kv_cols :] if s.gate else None
@@ -480,7 +481,7 @@ class LatentAttention(nn.Module):
             s.heads, gate=gate, out_dtype=self.dtype, sink=self.sink,
             window=s.window,
         )
-        o = ops.head_matmul_rope(o_lat, self.uv_t, s.heads)
+        o = ops.head_matmul_rope(o_lat, self.uv, s.heads)
         return F.linear(o, self.o_proj)
 
 

@@ -142,7 +142,7 @@ class VoboraxForCausalLM(nn.Module):
                 p.fill_(1.0)
             elif p.dim() >= 2:
                 # keep activations O(1) through the stack
-                fan_in = p.shape[-2] if leaf in ("uk", "uv_t") else p.shape[-1]
+                fan_in = p.shape[-2] if leaf == "uk_t" else p.shape[-1]
                 p.normal_(0.0, fan_in ** -0.5, generator=gen)
             else:
                 p.normal_(0.0, 0.1, generator=gen)

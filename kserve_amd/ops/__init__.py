@@ -636,11 +636,11 @@ def head_matmul_rope(
     out_dtype=None,
 ):
     """Per-head matrix product with an optional rotated tail:
-    x [T, heads*(k + tail)], w [heads, k, n] -> [T, heads*(n + tail)], the
+    x [T, heads*(k + tail)], w [heads, n, k] -> [T, heads*(n + tail)], the
     tail coordinates turned in pairs by the token's position."""
     out_dtype = out_dtype or x.dtype
     if x.is_cuda:
-        n = w.shape[2]
+        n = w.shape[1]
         out = torch.empty(
             (x.shape[0], heads * (n + tail)), dtype=out_dtype, device=x.device
         )

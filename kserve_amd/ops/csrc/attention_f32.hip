@@ -331,7 +331,7 @@ struct TileStage {
   }
 };
 
-template <typename T, int DP, int DVP, bool SPLITK>
+template <typename T, int DP, int DVP, bool SPLITK, bool VK>
 __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     T* __restrict__ out, const float* __restrict__ q,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -340,19 +340,27 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     const T* __restrict__ gate, long gate_stride, float scale, int heads,
     int kv_heads, int D, int DV, int block_size, int hpb,
     const float* __restrict__ sink, int chunk,
-    const float* __restrict__ out_inv_freq, int window, long v_row_stride) {
+    const float* __restrict__ out_inv_freq, int window, long v_row_stride,
+    float* __restrict__ ws) {
   extern __shared__ float lds[];
   constexpr int KS = DP + 4;   // K row stride: lanes of one MFMA read hit 64 banks
-  constexpr int VS = DVP + 4;  // V row stride: likewise for the 4-key-apart rows
+  // V row stride: likewise for the 4-key-apart rows. VK: the values are the
+  // leading columns of the key rows, so the staged K tile serves as V too
+  constexpr int VS = VK ? KS : DVP + 4;
   constexpr int ROWS = SPLITK ? 16 : 64;  // query rows per block
-  float* Ks = lds;             // [BK][KS]
-  float* Vs = Ks + BK * KS;    // [BK][VS]
+  float* Ks = lds;                       // [BK][KS]
+  float* Vs = VK ? Ks : Ks + BK * KS;    // [BK][VS]
 
   const int s = blockIdx.y;
   const int q0 = cu_q[s];
   const int q_len = cu_q[s + 1] - q0;
   const int tpb = ROWS / hpb;  // tokens per block
-  const int tok0 = blockIdx.x * tpb;
+  // decode: blockIdx.x numbers the key splits of the one token, and block
+  // x takes the tiles x, x + nsplit, ... of the visible keys
+  const int nsplit = SPLITK ? gridDim.x : 1;
+  const int split = SPLITK ? blockIdx.x : 0;
+  const int kstep = nsplit * BK;
+  const int tok0 = SPLITK ? 0 : blockIdx.x * tpb;
   if (tok0 >= q_len) return;
   const int head0 = blockIdx.z * hpb;
   const int g = head0 / (heads / kv_heads);
@@ -421,17 +429,20 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   // the next tile's global loads are in flight while this one is computed
   TileStage<T, DP> kst;
   TileStage<T, DVP> vst;
-  kst.fetch(k_cache, bt, kbeg, min(BK, last_pos + 1 - kbeg), g, kv_heads, D, D, block_size, bs_shift, kvec);
-  vst.fetch(v_cache, bt, kbeg, min(BK, last_pos + 1 - kbeg), g, kv_heads, DV, v_row_stride, block_size, bs_shift, vvec);
-  for (int k0 = kbeg; k0 <= last_pos; k0 += BK) {
+  const int kfirst = kbeg + split * BK;
+  kst.fetch(k_cache, bt, kfirst, min(BK, last_pos + 1 - kfirst), g, kv_heads, D, D, block_size, bs_shift, kvec);
+  if (!VK)
+    vst.fetch(v_cache, bt, kfirst, min(BK, last_pos + 1 - kfirst), g, kv_heads, DV, v_row_stride, block_size, bs_shift, vvec);
+  for (int k0 = kfirst; k0 <= last_pos; k0 += kstep) {
     __syncthreads();  // previous tile fully consumed
     kst.store(Ks);
-    vst.store(Vs);
+    if (!VK) vst.store(Vs);
     __syncthreads();
-    if (k0 + BK <= last_pos) {
-      const int nn = min(BK, last_pos + 1 - (k0 + BK));
-      kst.fetch(k_cache, bt, k0 + BK, nn, g, kv_heads, D, D, block_size, bs_shift, kvec);
-      vst.fetch(v_cache, bt, k0 + BK, nn, g, kv_heads, DV, v_row_stride, block_size, bs_shift, vvec);
+    if (k0 + kstep <= last_pos) {
+      const int nn = min(BK, last_pos + 1 - (k0 + kstep));
+      kst.fetch(k_cache, bt, k0 + kstep, nn, g, kv_heads, D, D, block_size, bs_shift, kvec);
+      if (!VK)
+        vst.fetch(v_cache, bt, k0 + kstep, nn, g, kv_heads, DV, v_row_stride, block_size, bs_shift, vvec);
     }
     if (k0 > wave_last || k0 + BK <= wave_first) continue;
 
@@ -530,6 +541,33 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     __syncthreads();
     // an element pair (dv, dv + DV/2) per thread when the output is turned
     // back, else one element
+    if (nsplit > 1) {
+      // partial (max, sum, weighted values) of this split, merged over the
+      // waves; ctx_attention_merge_kernel finishes. ws: per (seq, head,
+      // split) DV values, then max and sum.
+      for (int e = threadIdx.x; e < nrows * DV; e += NT) {
+        const int row = e / DV, dv = e % DV;
+        const int h2 = head0 + row % hpb;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) M = fmaxf(M, Ms[w * 16 + row]);
+        float L = 0.f, O = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+          const float mw = Ms[w * 16 + row];
+          const float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
+          L += Ls[w * 16 + row] * f;
+          O += Os[(w * 16 + row) * DVP + dv] * f;
+        }
+        float* wr = ws + (((long)s * heads + h2) * nsplit + split) * (DV + 2);
+        wr[dv] = O;
+        if (dv == 0) {
+          wr[DV] = M;
+          wr[DV + 1] = L;
+        }
+      }
+      return;
+    }
     const int ohalf = out_inv_freq ? DV / 2 : 0;
     const int per_row = out_inv_freq ? ohalf : DV;
     for (int e = threadIdx.x; e < nrows * per_row; e += NT) {
@@ -620,6 +658,44 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
     }
 }
 
+// Second pass of a split decode: one block per (sequence, head) combines the
+// splits' partials, adds the sink term, normalises and applies the gate.
+template <typename T>
+__global__ void ctx_attention_merge_kernel(
+    T* __restrict__ out, const float* __restrict__ ws,
+    const int* __restrict__ cu_q, const T* __restrict__ gate, long gate_stride,
+    const float* __restrict__ sink, int heads, int DV, int nsplit) {
+  const int s = blockIdx.x / heads, h = blockIdx.x % heads;
+  const int tok = cu_q[s];
+  if (cu_q[s + 1] - tok < 1) return;
+  const float* wr = ws + ((long)s * heads + h) * nsplit * (DV + 2);
+  float M = -INFINITY;
+  for (int i = 0; i < nsplit; ++i) M = fmaxf(M, wr[i * (DV + 2) + DV]);
+  float L = 0.f;
+  if (sink) {
+    const float sl = sink[h] * 1.44269504088896340736f;
+    M = fmaxf(M, sl);
+    L = exp2f(sl - M);
+  }
+  for (int i = 0; i < nsplit; ++i) {
+    const float mi = wr[i * (DV + 2) + DV];
+    if (mi != -INFINITY) L += wr[i * (DV + 2) + DV + 1] * exp2f(mi - M);
+  }
+  float f = 1.0f / L;
+  if (gate) {
+    const float gv = ld_f32(gate, (long)tok * gate_stride + h);
+    f *= 1.0f / (1.0f + expf(-gv));
+  }
+  for (int dv = threadIdx.x; dv < DV; dv += blockDim.x) {
+    float O = 0.f;
+    for (int i = 0; i < nsplit; ++i) {
+      const float mi = wr[i * (DV + 2) + DV];
+      if (mi != -INFINITY) O += wr[i * (DV + 2) + dv] * exp2f(mi - M);
+    }
+    st_f32(out, ((long)tok * heads + h) * DV + dv, O * f);
+  }
+}
+
 }  // namespace
 
 extern "C" hipError_t ks_qk_norm_temp_cache(
@@ -690,78 +766,112 @@ extern "C" hipError_t ks_qk_headnorm_rope_cache(
   return hipSuccess;
 }
 
-template <typename T, int DP, int DVP>
-hipError_t launch_ctx_attention(void* out, const void* q, const void* k_cache,
-                                const void* v_cache, const void* block_tables,
-                                int bt_stride, const void* cu_q,
-                                const void* ctx_lens, const void* gate,
-                                long gate_stride, float scale, int num_seqs,
-                                int max_q_len, int heads, int kv_heads, int D,
-                                int DV, int block_size, const void* sink,
-                                int chunk, const void* out_inv_freq,
-                                int window, long v_row_stride,
-                                hipStream_t stream) {
-  size_t smem = sizeof(float) * (size_t)BK * (DP + 4 + DVP + 4);
-  const bool decode = max_q_len == 1;
-  // decode: one token per sequence, a block takes heads of one group
+// decode: one token per sequence, a block takes up to 16 heads of one group
+static int decode_heads_per_block(int heads, int kv_heads) {
+  const int gs = heads / kv_heads;
+  int hpb = 1;
+  for (int c = 1; c <= 16 && c <= gs; ++c)
+    if (gs % c == 0) hpb = c;
+  return hpb;
+}
+
+// Key splits of a decode launch: enough blocks to put several on every
+// compute unit (a block runs few waves and waits on its tile loads), no more
+// than 8, and with a window no more than the window has tiles. It cannot
+// depend on the context lengths, which only the device knows: a split
+// without keys writes an empty partial.
+extern "C" int ks_ctx_attention_decode_splits(int num_seqs, int heads,
+                                              int kv_heads, int window,
+                                              int has_out_rotation) {
+  if (has_out_rotation) return 1;
+  const int blocks = num_seqs * (heads / decode_heads_per_block(heads, kv_heads));
+  int n = cdiv(1024, blocks > 0 ? blocks : 1);
+  if (n > 8) n = 8;
+  if (window > 0 && n > cdiv(window, BK)) n = cdiv(window, BK);
+  return n < 1 ? 1 : n;
+}
+
+struct CtxArgs {
+  void* out;
+  const void *q, *k_cache, *v_cache, *block_tables;
+  int bt_stride;
+  const void *cu_q, *ctx_lens, *gate;
+  long gate_stride;
+  float scale;
+  int num_seqs, max_q_len, heads, kv_heads, D, DV, block_size;
+  const void* sink;
+  int chunk;
+  const void* out_inv_freq;
+  int window;
+  long v_row_stride;
+  void* ws;
+  int nsplit;
+  hipStream_t stream;
+};
+
+template <typename T, int DP, int DVP, bool VK>
+hipError_t launch_ctx_attention(const CtxArgs& a) {
+  size_t smem = sizeof(float) * (size_t)BK * (DP + 4 + (VK ? 0 : DVP + 4));
+  const bool decode = a.max_q_len == 1;
   int hpb = 1;
   if (decode) {
-    const int gs = heads / kv_heads;
-    for (int c = 1; c <= 16 && c <= gs; ++c)
-      if (gs % c == 0) hpb = c;
+    hpb = decode_heads_per_block(a.heads, a.kv_heads);
     const size_t merge = sizeof(float) * (size_t)NW * 16 * (DVP + 2);
     if (merge > smem) smem = merge;
   }
   const int rows = decode ? 16 : 64;
-  dim3 grid(cdiv(max_q_len, rows / hpb), num_seqs, heads / hpb);
-  auto fn = decode ? ctx_attention_f32_kernel<T, DP, DVP, true>
-                   : ctx_attention_f32_kernel<T, DP, DVP, false>;
+  const int nsplit = decode ? a.nsplit : 1;
+  dim3 grid(decode ? nsplit : cdiv(a.max_q_len, rows / hpb), a.num_seqs,
+            a.heads / hpb);
+  auto fn = decode ? ctx_attention_f32_kernel<T, DP, DVP, true, VK>
+                   : ctx_attention_f32_kernel<T, DP, DVP, false, VK>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(
         (const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(fn, grid, dim3(NT), smem, stream, (T*)out, (const float*)q,
-                     (const T*)k_cache, (const T*)v_cache,
-                     (const int*)block_tables, bt_stride, (const int*)cu_q,
-                     (const int*)ctx_lens, (const T*)gate, gate_stride, scale,
-                     heads, kv_heads, D, DV, block_size, hpb,
-                     (const float*)sink, chunk, (const float*)out_inv_freq,
-                     window, v_row_stride);
+  hipLaunchKernelGGL(fn, grid, dim3(NT), smem, a.stream, (T*)a.out,
+                     (const float*)a.q, (const T*)a.k_cache,
+                     (const T*)a.v_cache, (const int*)a.block_tables,
+                     a.bt_stride, (const int*)a.cu_q, (const int*)a.ctx_lens,
+                     (const T*)a.gate, a.gate_stride, a.scale, a.heads,
+                     a.kv_heads, a.D, a.DV, a.block_size, hpb,
+                     (const float*)a.sink, a.chunk,
+                     (const float*)a.out_inv_freq, a.window, a.v_row_stride,
+                     (float*)a.ws);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || nsplit <= 1) return e;
+  hipLaunchKernelGGL(ctx_attention_merge_kernel<T>,
+                     dim3(a.num_seqs * a.heads), dim3(64), 0, a.stream,
+                     (T*)a.out, (const float*)a.ws, (const int*)a.cu_q,
+                     (const T*)a.gate, a.gate_stride, (const float*)a.sink,
+                     a.heads, a.DV, nsplit);
   return hipGetLastError();
 }
 
-#define CTX_ARGS                                                              \
-  out, q, k_cache, v_cache, block_tables, bt_stride, cu_q, ctx_lens, gate,    \
-      gate_stride, scale, num_seqs, max_q_len, heads, kv_heads, D, DV,        \
-      block_size, sink, chunk, out_inv_freq, window, v_row_stride, stream
+template <typename T, int DP, int DVP>
+hipError_t dispatch_vk(const CtxArgs& a) {
+  // the values are the leading columns of the key rows themselves
+  const bool vk = a.v_cache == a.k_cache && a.v_row_stride == a.D && DVP <= DP;
+  if constexpr (DVP <= DP) {
+    if (vk) return launch_ctx_attention<T, DP, DVP, true>(a);
+  }
+  return launch_ctx_attention<T, DP, DVP, false>(a);
+}
 
 template <typename T, int DP>
-hipError_t dispatch_dv(void* out, const void* q, const void* k_cache,
-                       const void* v_cache, const void* block_tables,
-                       int bt_stride, const void* cu_q, const void* ctx_lens,
-                       const void* gate, long gate_stride, float scale,
-                       int num_seqs, int max_q_len, int heads, int kv_heads,
-                       int D, int DV, int block_size, const void* sink,
-                       int chunk, const void* out_inv_freq, int window,
-                       long v_row_stride, hipStream_t stream) {
-  if (DV <= 64) return launch_ctx_attention<T, DP, 64>(CTX_ARGS);
-  if (DV <= 128) return launch_ctx_attention<T, DP, 128>(CTX_ARGS);
-  return launch_ctx_attention<T, DP, 256>(CTX_ARGS);
+hipError_t dispatch_dv(const CtxArgs& a) {
+  if (a.DV <= 64) return dispatch_vk<T, DP, 64>(a);
+  if (a.DV <= 128) return dispatch_vk<T, DP, 128>(a);
+  if (a.DV <= 192) return dispatch_vk<T, DP, 192>(a);
+  return dispatch_vk<T, DP, 256>(a);
 }
 
 template <typename T>
-hipError_t dispatch_d(void* out, const void* q, const void* k_cache,
-                      const void* v_cache, const void* block_tables,
-                      int bt_stride, const void* cu_q, const void* ctx_lens,
-                      const void* gate, long gate_stride, float scale,
-                      int num_seqs, int max_q_len, int heads, int kv_heads,
-                      int D, int DV, int block_size, const void* sink,
-                      int chunk, const void* out_inv_freq, int window,
-                      long v_row_stride, hipStream_t stream) {
-  if (D <= 64) return dispatch_dv<T, 64>(CTX_ARGS);
-  if (D <= 128) return dispatch_dv<T, 128>(CTX_ARGS);
-  return dispatch_dv<T, 256>(CTX_ARGS);
+hipError_t dispatch_d(const CtxArgs& a) {
+  if (a.D <= 64) return dispatch_dv<T, 64>(a);
+  if (a.D <= 128) return dispatch_dv<T, 128>(a);
+  return dispatch_dv<T, 256>(a);
 }
 
 extern "C" hipError_t ks_ctx_attention_f32(
@@ -770,13 +880,18 @@ extern "C" hipError_t ks_ctx_attention_f32(
     const void* ctx_lens, const void* gate, long gate_stride, float scale,
     int num_seqs, int max_q_len, int heads, int kv_heads, int D, int DV,
     int block_size, int is_f32, const void* sink, int chunk,
-    const void* out_inv_freq, int window, long v_row_stride,
-    hipStream_t stream) {
+    const void* out_inv_freq, int window, long v_row_stride, void* ws,
+    int nsplit, hipStream_t stream) {
   if (num_seqs == 0 || max_q_len == 0) return hipSuccess;
   if (D < 1 || D > 256 || DV < 1 || DV > 256 || kv_heads < 1 ||
       heads % kv_heads != 0 || chunk < 0 || window < 0 ||
       (chunk > 0 && window > 0) || v_row_stride < DV ||
-      (out_inv_freq && DV % 2 != 0))
+      (out_inv_freq && DV % 2 != 0) || nsplit < 1 || (nsplit > 1 && !ws) ||
+      (nsplit > 1 && out_inv_freq))
     return hipErrorInvalidValue;
-  return is_f32 ? dispatch_d<float>(CTX_ARGS) : dispatch_d<short>(CTX_ARGS);
+  const CtxArgs a{out, q, k_cache, v_cache, block_tables, bt_stride, cu_q,
+                  ctx_lens, gate, gate_stride, scale, num_seqs, max_q_len,
+                  heads, kv_heads, D, DV, block_size, sink, chunk,
+                  out_inv_freq, window, v_row_stride, ws, nsplit, stream};
+  return is_f32 ? dispatch_d<float>(a) : dispatch_d<short>(a);
 }

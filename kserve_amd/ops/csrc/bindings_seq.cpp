@@ -31,7 +31,9 @@ hipError_t ks_ctx_attention_f32(void*, const void*, const void*, const void*,
                                 const void*, int, const void*, const void*,
                                 const void*, long, float, int, int, int, int,
                                 int, int, int, int, const void*, int,
-                                const void*, int, long, hipStream_t);
+                                const void*, int, long, void*, int,
+                                hipStream_t);
+int ks_ctx_attention_decode_splits(int, int, int, int, int);
 hipError_t ks_qk_headnorm_rope_cache(void*, const void*, const void*,
                                      const void*, long, const void*,
                                      const void*, const void*, const void*,
@@ -355,13 +357,26 @@ void ctx_attention_f32(at::Tensor& out, at::Tensor& q, at::Tensor& k_cache,
   }
   TORCH_CHECK(chunk >= 0 && window >= 0 && !(chunk > 0 && window > 0),
               "chunk / window: not negative, at most one of them");
+  // a decode batch splits every sequence's keys over several blocks, which
+  // leave partial results in a scratch tensor for a merge pass
+  int nsplit = 1;
+  at::Tensor ws;
+  if (max_q_len == 1) {
+    nsplit = ks_ctx_attention_decode_splits(num_seqs, (int)heads, G,
+                                            (int)window, fp != nullptr);
+    if (nsplit > 1)
+      ws = at::empty({(int64_t)num_seqs * heads * nsplit * (DV + 2)},
+                     q.options().dtype(at::kFloat));
+  }
   check_hip(ks_ctx_attention_f32(
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                 v_cache.data_ptr(), block_tables.data_ptr(),
                 (int)block_tables.stride(0), cu_q.data_ptr(),
                 ctx_lens.data_ptr(), gp, gst, (float)scale, num_seqs,
                 (int)max_q_len, (int)heads, G, D, DV, bs, f32, sp, (int)chunk,
-                fp, (int)window, (long)vrs, current_stream()),
+                fp, (int)window, (long)vrs,
+                nsplit > 1 ? ws.data_ptr() : nullptr, nsplit,
+                current_stream()),
             "ctx_attention_f32");
 }
 
@@ -726,9 +741,9 @@ void head_matmul_rope(at::Tensor& out, at::Tensor& x, at::Tensor& w,
                       const c10::optional<at::Tensor>& inv_freq) {
   CHECK_ROWS(x);
   TORCH_CHECK(w.dim() == 3 && w.is_contiguous() && w.size(0) == heads,
-              "w [heads, k, n] contiguous");
+              "w [heads, n, k] contiguous");
   const int in_f32 = act_is_f32(x, "x"), out_f32 = act_is_f32(out, "out");
-  const int tokens = x.size(0), K = w.size(1), N = w.size(2);
+  const int tokens = x.size(0), N = w.size(1), K = w.size(2);
   TORCH_CHECK(act_is_f32(w, "w") == in_f32 && (out_f32 || !in_f32) &&
                   tail >= 0 && x.size(1) == heads * (K + tail) &&
                   out.is_contiguous() &&

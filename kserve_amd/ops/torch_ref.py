@@ -701,14 +701,14 @@ def latent_norm_rope_cache(
 def head_matmul_rope(
     x, w, heads: int, tail: int, positions, inv_freq, out_dtype
 ):
-    """x [T, heads * (k + tail)], w [heads, k, n] -> [T, heads * (n + tail)]:
-    per head the first k coordinates times the head's matrix (fp32 sums),
+    """x [T, heads * (k + tail)], w [heads, n, k] -> [T, heads * (n + tail)]:
+    per head the head's matrix times the first k coordinates (fp32 sums),
     followed by the ``tail`` coordinates rotated in pairs by the token's
     position (copied when ``inv_freq`` is None)."""
     T = x.shape[0]
-    H, k, n = w.shape
+    H, n, k = w.shape
     xh = x.reshape(T, heads, k + tail).float()
-    y = torch.einsum("thk,hkn->thn", xh[..., :k], w.float())
+    y = torch.einsum("thk,hnk->thn", xh[..., :k], w.float())
     if tail:
         y = torch.cat([y, rotate_pairs(xh[..., k:], positions, inv_freq)], dim=-1)
     return y.reshape(T, heads * (n + tail)).to(out_dtype)

@@ -572,8 +572,8 @@ class TestConfigAndRegistry:
         assert torch.equal(a.in_proj[:20], sd["l0.mix.dq"].float())
         assert torch.equal(a.in_proj[20:52], sd["l0.mix.dkv"].float())
         assert torch.equal(a.in_proj[52:], sd["l0.mix.g"].float())
-        assert torch.equal(a.uk[2], sd["l0.mix.uk"].float()[32:48])
-        assert torch.equal(a.uv_t[1], sd["l0.mix.uv"].float()[8:16].T)
+        assert torch.equal(a.uk_t[2], sd["l0.mix.uk"].float()[32:48].T)
+        assert torch.equal(a.uv[1], sd["l0.mix.uv"].float()[8:16])
         assert torch.equal(model.layers[2].attn.sink, sd["l2.mix.sink"].float())
         m = model.layers[1].mlp
         assert torch.equal(m.gate_up[4, 10:], sd["l1.mlp.e4.up"].float())

@@ -163,16 +163,17 @@ class TestHeadMatmulRope:
     @pytest.mark.parametrize(
         "T,H,K,N,tail,rot_dims",
         [(5, 3, 16, 24, 8, 8), (70, 2, 40, 300, 0, 0), (33, 5, 64, 96, 32, 32),
-         (1, 4, 24, 70, 10, 6), (64, 1, 130, 64, 0, 0)],
+         (1, 4, 24, 70, 10, 6), (64, 1, 130, 64, 0, 0), (200, 3, 72, 100, 0, 0),
+         (2100, 2, 128, 192, 64, 64), (130, 2, 20, 36, 4, 4), (300, 1, 96, 80, 0, 0)],
     )
     def test_against_oracle(self, be, T, H, K, N, tail, rot_dims):
         base = 5000.0
         x = rnd(T, H * (K + tail), seed=21, dtype=be[1])
-        w = rnd(H, K, N, seed=22, scale=K ** -0.5, dtype=be[1])
-        pos = torch.arange(T) * 37 % 1001
+        w = rnd(H, N, K, seed=22, scale=K ** -0.5, dtype=be[1])
+        pos = torch.arange(T) * 37 % 257   # fp32 angles: keep them small
         inv = rotary_inv_freq(rot_dims, base) if rot_dims else None
         xh = x.double().view(T, H, K + tail)
-        want = torch.einsum("thk,hkn->thn", xh[..., :K], w.double())
+        want = torch.einsum("thk,hnk->thn", xh[..., :K], w.double())
         if tail:
             tl = xh[..., K:]
             if rot_dims:
