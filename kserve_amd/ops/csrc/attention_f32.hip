@@ -406,12 +406,39 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   // lg stands for d = lg * DP/4 + ks, so a lane's K values are contiguous in
   // LDS (16-byte reads) and so are its q values here. Pre-multiplied by the
   // softmax scale and log2(e): the softmax runs on exp2.
+  // The block's query rows go through LDS first (rows of D contiguous
+  // floats, read by consecutive lanes; zero past D and past the last row),
+  // where the K tile will be staged afterwards: a lane's own values are 64
+  // floats apart from its neighbour's, which global memory serves badly.
   const float qscale = scale * 1.44269504088896340736f;
   float qf[DP / 4];
+  {
+    float* Qs = lds;  // [ROWS][KS]
+    for (int e = threadIdx.x; e < ROWS * (DP / 4); e += NT) {
+      const int rr = e / (DP / 4), d = (e % (DP / 4)) * 4;
+      f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (rr < nrows) {
+        const float* src =
+            q + ((long)(q0 + tok0 + rr / hpb) * heads + head0 + rr % hpb) * D;
+        if ((D % 4) == 0 && d + 3 < D) {
+          v = *reinterpret_cast<const f32x4*>(src + d);
+        } else {
 #pragma unroll
-  for (int ks = 0; ks < DP / 4; ++ks) {
-    const int d = lg * (DP / 4) + ks;
-    qf[ks] = (row_ok && d < D) ? q[((long)tok * heads + hd) * D + d] * qscale : 0.f;
+          for (int c = 0; c < 4; ++c)
+            if (d + c < D) v[c] = src[d + c];
+        }
+      }
+      *reinterpret_cast<f32x4*>(Qs + rr * KS + d) = v * qscale;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k4 = 0; k4 < DP / 16; ++k4) {
+      const f32x4 v =
+          *reinterpret_cast<const f32x4*>(Qs + r * KS + lg * (DP / 4) + 4 * k4);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) qf[4 * k4 + c] = v[c];
+    }
+    // the first K tile is stored behind the loop's own barrier
   }
   f32x4 o[DVP / 16];
 #pragma unroll
