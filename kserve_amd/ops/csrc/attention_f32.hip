@@ -38,6 +38,8 @@
 //    partial (max, sum, O) through LDS at the end, so the group's K/V is read
 //    once. Head sizes are padded up to 64/128/256 with zeros. An optional
 //    per-(token, head) gate multiplies the result by sigmoid(gate).
+#include <type_traits>
+
 #include "dtype_io.h"
 
 namespace {
@@ -289,7 +291,9 @@ struct Chunk8<float> {
 
 // rows [k0, k0 + nk) of one kv head, WP (padded width) columns: each thread
 // owns WP / 32 chunks of 8; fetch() issues the global loads, store() writes
-// them to LDS as fp32 [BK][WP + 4], zero past the head size and past nk
+// them to LDS in the cache dtype as [BK][WP + 4], zero past the head size and
+// past nk. A bf16 tile is widened when the matrix-core operands are read
+// (lds4): half the LDS of an fp32 tile, so twice the blocks per compute unit.
 template <typename T, int WP>
 struct TileStage {
   static constexpr int CPR = WP / 8;          // chunks per row
@@ -329,7 +333,28 @@ struct TileStage {
       o[1] = f32x4{ch[i].get(4), ch[i].get(5), ch[i].get(6), ch[i].get(7)};
     }
   }
+  // rows are 8-byte aligned only (LS = WP + 4 elements): two 8-byte stores
+  __device__ __forceinline__ void store(short* dst) const {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + NT * i;
+      const int j = c / CPR, d0 = (c % CPR) * 8;
+      short4_t* o = reinterpret_cast<short4_t*>(dst + j * LS + d0);
+      o[0] = short4_t{ch[i].x[0], ch[i].x[1], ch[i].x[2], ch[i].x[3]};
+      o[1] = short4_t{ch[i].x[4], ch[i].x[5], ch[i].x[6], ch[i].x[7]};
+    }
+  }
 };
+
+// four consecutive tile elements as fp32
+__device__ __forceinline__ f32x4 lds4(const float* p) {
+  return *reinterpret_cast<const f32x4*>(p);
+}
+__device__ __forceinline__ f32x4 lds4(const short* p) {
+  const short4_t x = *reinterpret_cast<const short4_t*>(p);
+  return f32x4{bf16_bits_to_float(x[0]), bf16_bits_to_float(x[1]),
+               bf16_bits_to_float(x[2]), bf16_bits_to_float(x[3])};
+}
 
 template <typename T, int DP, int DVP, bool SPLITK, bool VK>
 __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
@@ -348,8 +373,14 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   // leading columns of the key rows, so the staged K tile serves as V too
   constexpr int VS = VK ? KS : DVP + 4;
   constexpr int ROWS = SPLITK ? 16 : 64;  // query rows per block
-  float* Ks = lds;                       // [BK][KS]
-  float* Vs = VK ? Ks : Ks + BK * KS;    // [BK][VS]
+  // Staged tiles: fp32 in prefill (widened once when stored; every wave
+  // reads the whole tile), the cache dtype in decode (widened when the
+  // operands are read; each wave reads a quarter of the tile, and half the
+  // LDS means twice the blocks per compute unit, which is what a decode block
+  // waiting on its tile loads needs).
+  using TL = typename std::conditional<SPLITK, T, float>::type;
+  TL* Ks = reinterpret_cast<TL*>(lds);   // [BK][KS]
+  TL* Vs = VK ? Ks : Ks + BK * KS;       // [BK][VS]
 
   const int s = blockIdx.y;
   const int q0 = cu_q[s];
@@ -406,14 +437,16 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   // lg stands for d = lg * DP/4 + ks, so a lane's K values are contiguous in
   // LDS (16-byte reads) and so are its q values here. Pre-multiplied by the
   // softmax scale and log2(e): the softmax runs on exp2.
-  // The block's query rows go through LDS first (rows of D contiguous
-  // floats, read by consecutive lanes; zero past D and past the last row),
-  // where the K tile will be staged afterwards: a lane's own values are 64
-  // floats apart from its neighbour's, which global memory serves badly.
+  // Q^T fragments, pre-multiplied by the softmax scale and log2(e) (the
+  // softmax runs on exp2). The block's query rows go through LDS first (rows
+  // of D contiguous floats, read by consecutive lanes; zero past D and past
+  // the last row), where the K tile is staged afterwards: a lane's own
+  // values are 64 floats apart from its neighbour's, which global memory
+  // serves badly.
   const float qscale = scale * 1.44269504088896340736f;
   float qf[DP / 4];
   {
-    float* Qs = lds;  // [ROWS][KS]
+    float* Qs = lds;  // [ROWS][KS] floats
     for (int e = threadIdx.x; e < ROWS * (DP / 4); e += NT) {
       const int rr = e / (DP / 4), d = (e % (DP / 4)) * 4;
       f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -487,8 +520,7 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
 #pragma unroll
       for (int t = 0; t < KT; ++t) {
         const int kt = SPLITK ? wave : t;
-        const f32x4 kv = *reinterpret_cast<const f32x4*>(
-            Ks + (16 * kt + li) * KS + lg * (DP / 4) + 4 * k4);
+        const f32x4 kv = lds4(Ks + (16 * kt + li) * KS + lg * (DP / 4) + 4 * k4);
         sc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[0], qf[4 * k4 + 0], sc[t], 0, 0, 0);
         sc2[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[1], qf[4 * k4 + 1], sc2[t], 0, 0, 0);
         sc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[2], qf[4 * k4 + 2], sc[t], 0, 0, 0);
@@ -536,12 +568,11 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
       for (int v = 0; v < 4; ++v) {
         // row li of output tile i is value column 64 (i/4) + 4 li + i%4: the
         // four tiles of a 64-column block come from one 16-byte read
-        const f32x4* va = reinterpret_cast<const f32x4*>(
-            Vs + (16 * kt + 4 * lg + v) * VS + 4 * li);
+        const TL* va = Vs + (16 * kt + 4 * lg + v) * VS + 4 * li;
         const float pb = sc[t][v];
 #pragma unroll
         for (int j = 0; j < DVP / 64; ++j) {
-          const f32x4 vv = va[16 * j];
+          const f32x4 vv = lds4(va + 64 * j);
 #pragma unroll
           for (int c = 0; c < 4; ++c)
             o[4 * j + c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[c], pb, o[4 * j + c], 0, 0, 0);
@@ -551,7 +582,12 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
   }
 
   if (SPLITK) {
-    // merge the four waves' partial results: Ms/Ls [NW][16], Os [NW][16][DVP]
+    // merge the four waves' partial results: Ms/Ls [NW][16], Os [NW][16][pw].
+    // Value columns go through LDS in passes of pw columns (two passes of
+    // 128 for wider values, which bounds the block's LDS; one pass when the
+    // output is turned back, since a pair spans both halves of the row).
+    const int np = (DVP <= 128 || out_inv_freq) ? 1 : 2;
+    const int pw = np == 1 ? DVP : 128;
     __syncthreads();
     float* Ms = lds;
     float* Ls = Ms + NW * 16;
@@ -560,78 +596,85 @@ __global__ void __launch_bounds__(NT) ctx_attention_f32_kernel(
       Ms[wave * 16 + li] = m;
       Ls[wave * 16 + li] = l;
     }
+    for (int p = 0; p < np; ++p) {
+      const int c0 = p * pw, c1 = min(DV, c0 + pw);
+      if (p) __syncthreads();  // the previous pass has been read
 #pragma unroll
-    for (int i = 0; i < DVP / 16; ++i)
+      for (int i = 0; i < DVP / 16; ++i)
+        if (64 * (i / 4) / pw == p) {
 #pragma unroll
-      for (int v = 0; v < 4; ++v)
-        Os[(wave * 16 + li) * DVP + 64 * (i / 4) + 4 * (4 * lg + v) + i % 4] = o[i][v];
-    __syncthreads();
-    // an element pair (dv, dv + DV/2) per thread when the output is turned
-    // back, else one element
-    if (nsplit > 1) {
-      // partial (max, sum, weighted values) of this split, merged over the
-      // waves; ctx_attention_merge_kernel finishes. ws: per (seq, head,
-      // split) DV values, then max and sum.
-      for (int e = threadIdx.x; e < nrows * DV; e += NT) {
-        const int row = e / DV, dv = e % DV;
-        const int h2 = head0 + row % hpb;
+          for (int v = 0; v < 4; ++v)
+            Os[(wave * 16 + li) * pw + 64 * (i / 4) - c0 + 4 * (4 * lg + v) + i % 4] = o[i][v];
+        }
+      __syncthreads();
+      if (nsplit > 1) {
+        // partial (max, sum, weighted values) of this split, merged over the
+        // waves; ctx_attention_merge_kernel finishes. ws: per (seq, head,
+        // split) DV values, then max and sum.
+        const int cw = c1 - c0;
+        for (int e = threadIdx.x; e < nrows * cw; e += NT) {
+          const int row = e / cw, dv = c0 + e % cw;
+          const int h2 = head0 + row % hpb;
+          float M = -INFINITY;
+#pragma unroll
+          for (int w = 0; w < NW; ++w) M = fmaxf(M, Ms[w * 16 + row]);
+          float L = 0.f, O = 0.f;
+#pragma unroll
+          for (int w = 0; w < NW; ++w) {
+            const float mw = Ms[w * 16 + row];
+            const float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
+            L += Ls[w * 16 + row] * f;
+            O += Os[(w * 16 + row) * pw + dv - c0] * f;
+          }
+          float* wr = ws + (((long)s * heads + h2) * nsplit + split) * (DV + 2);
+          wr[dv] = O;
+          if (dv == 0) {
+            wr[DV] = M;
+            wr[DV + 1] = L;
+          }
+        }
+        continue;
+      }
+      // an element pair (dv, dv + DV/2) per thread when the output is turned
+      // back (one pass), else one element
+      const int ohalf = out_inv_freq ? DV / 2 : 0;
+      const int per_row = out_inv_freq ? ohalf : c1 - c0;
+      for (int e = threadIdx.x; e < nrows * per_row; e += NT) {
+        const int row = e / per_row, dv = c0 + e % per_row;
+        const int tk = q0 + tok0 + row / hpb, h2 = head0 + row % hpb;
         float M = -INFINITY;
 #pragma unroll
         for (int w = 0; w < NW; ++w) M = fmaxf(M, Ms[w * 16 + row]);
-        float L = 0.f, O = 0.f;
+        float L = 0.f;
+        if (sink) {
+          const float sl = sink[h2] * 1.44269504088896340736f;
+          M = fmaxf(M, sl);
+          L = exp2f(sl - M);
+        }
+        float O = 0.f, O2 = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
           const float mw = Ms[w * 16 + row];
           const float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
           L += Ls[w * 16 + row] * f;
-          O += Os[(w * 16 + row) * DVP + dv] * f;
+          O += Os[(w * 16 + row) * pw + dv - c0] * f;
+          if (out_inv_freq) O2 += Os[(w * 16 + row) * pw + dv + ohalf] * f;
         }
-        float* wr = ws + (((long)s * heads + h2) * nsplit + split) * (DV + 2);
-        wr[dv] = O;
-        if (dv == 0) {
-          wr[DV] = M;
-          wr[DV + 1] = L;
+        float f = 1.0f / L;
+        if (gate) {
+          const float gv = ld_f32(gate, (long)tk * gate_stride + h2);
+          f *= 1.0f / (1.0f + expf(-gv));
         }
-      }
-      return;
-    }
-    const int ohalf = out_inv_freq ? DV / 2 : 0;
-    const int per_row = out_inv_freq ? ohalf : DV;
-    for (int e = threadIdx.x; e < nrows * per_row; e += NT) {
-      const int row = e / per_row, dv = e % per_row;
-      const int tk = q0 + tok0 + row / hpb, h2 = head0 + row % hpb;
-      float M = -INFINITY;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) M = fmaxf(M, Ms[w * 16 + row]);
-      float L = 0.f;
-      if (sink) {
-        const float sl = sink[h2] * 1.44269504088896340736f;
-        M = fmaxf(M, sl);
-        L = exp2f(sl - M);
-      }
-      float O = 0.f, O2 = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) {
-        const float mw = Ms[w * 16 + row];
-        const float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
-        L += Ls[w * 16 + row] * f;
-        O += Os[(w * 16 + row) * DVP + dv] * f;
-        if (out_inv_freq) O2 += Os[(w * 16 + row) * DVP + dv + ohalf] * f;
-      }
-      float f = 1.0f / L;
-      if (gate) {
-        const float gv = ld_f32(gate, (long)tk * gate_stride + h2);
-        f *= 1.0f / (1.0f + expf(-gv));
-      }
-      O *= f;
-      if (out_inv_freq) {
-        O2 *= f;
-        float sn, cs;
-        sincosf((float)(base_pos + row / hpb) * out_inv_freq[dv], &sn, &cs);
-        st_f32(out, ((long)tk * heads + h2) * DV + dv, O * cs + O2 * sn);
-        st_f32(out, ((long)tk * heads + h2) * DV + dv + ohalf, O2 * cs - O * sn);
-      } else {
-        st_f32(out, ((long)tk * heads + h2) * DV + dv, O);
+        O *= f;
+        if (out_inv_freq) {
+          O2 *= f;
+          float sn, cs;
+          sincosf((float)(base_pos + row / hpb) * out_inv_freq[dv], &sn, &cs);
+          st_f32(out, ((long)tk * heads + h2) * DV + dv, O * cs + O2 * sn);
+          st_f32(out, ((long)tk * heads + h2) * DV + dv + ohalf, O2 * cs - O * sn);
+        } else {
+          st_f32(out, ((long)tk * heads + h2) * DV + dv, O);
+        }
       }
     }
     return;
@@ -838,13 +881,23 @@ struct CtxArgs {
 
 template <typename T, int DP, int DVP, bool VK>
 hipError_t launch_ctx_attention(const CtxArgs& a) {
-  size_t smem = sizeof(float) * (size_t)BK * (DP + 4 + (VK ? 0 : DVP + 4));
+  // the staged tiles are fp32 in prefill and in the cache dtype in decode;
+  // the other uses of the same LDS (query rows; decode: cross-wave merge;
+  // prefill: rows to turn back) are fp32
   const bool decode = a.max_q_len == 1;
+  size_t smem = (decode ? sizeof(T) : sizeof(float)) * (size_t)BK *
+                (DP + 4 + (VK ? 0 : DVP + 4));
   int hpb = 1;
   if (decode) {
     hpb = decode_heads_per_block(a.heads, a.kv_heads);
-    const size_t merge = sizeof(float) * (size_t)NW * 16 * (DVP + 2);
+    const int pw = (DVP <= 128 || a.out_inv_freq) ? DVP : 128;
+    const size_t merge = sizeof(float) * (size_t)NW * 16 * (pw + 2);
+    const size_t qrows = sizeof(float) * (size_t)16 * (DP + 4);
     if (merge > smem) smem = merge;
+    if (qrows > smem) smem = qrows;
+  } else if (a.out_inv_freq) {
+    const size_t rows = sizeof(float) * (size_t)64 * (DVP + 1);
+    if (rows > smem) smem = rows;
   }
   const int rows = decode ? 16 : 64;
   const int nsplit = decode ? a.nsplit : 1;
