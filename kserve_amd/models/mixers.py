@@ -400,9 +400,17 @@ class LatentAttention(nn.Module):
     Options: ``window`` (sliding), ``sink`` (softmax denominator term),
     ``gate``, ``rot_dim`` = 0 (no positions at all), ``kv_from`` (no kv
     projection: the layer attends to the pages of an earlier layer with its
-    own U_k / U_v)."""
+    own U_k / U_v).
 
-    # widest cached row the fp32 attention kernel takes
+    Rows wider than the attention kernel takes (``MAX_CACHE_DIM``) switch the
+    layer to the expanded form: every step reads the sequences' cached rows,
+    expands them to per-head keys [unrotated | shared rotated part] and values
+    in scratch pages, and runs the same kernel as plain multi-head attention.
+    That costs a pass over the whole context per step and a host read of the
+    context lengths, so such a model decodes without captured graphs; it is
+    there so that any size runs."""
+
+    # widest cached row (and widest head) the fp32 attention kernel takes
     MAX_CACHE_DIM = 256
 
     def __init__(self, width: int, spec: LatentAttentionSpec, eps: float, dtype):
@@ -413,10 +421,11 @@ class LatentAttention(nn.Module):
         s = spec
         if s.rot_dims % 2 or s.rot_dims > s.rot_dim:
             raise ValueError("rotated coordinates: even, at most the rotated part")
-        if s.cache_dim > self.MAX_CACHE_DIM:
+        self.expanded = s.cache_dim > self.MAX_CACHE_DIM
+        if self.expanded and max(s.dim + s.rot_dim, s.vdim) > self.MAX_CACHE_DIM:
             raise NotImplementedError(
-                f"latent row of {s.cache_dim} columns (kv_rank + rot_dim): the "
-                f"attention kernel takes at most {self.MAX_CACHE_DIM}"
+                f"heads of {s.dim + s.rot_dim} key / {s.vdim} value columns: "
+                f"the attention kernel takes at most {self.MAX_CACHE_DIM}"
             )
         self.own_kv = s.kv_from is None
         self.kv_cols = s.cache_dim if self.own_kv else 0
@@ -470,11 +479,16 @@ class LatentAttention(nn.Module):
             self.eps, self.inv_freq,
         )
         q = F.linear(cq, self.uq)
+        gate = proj[:, s.q_rank + self.kv_cols :] if s.gate else None
+        if self.expanded:
+            return F.linear(
+                self._expanded_attention(q, gate, positions, cache, meta),
+                self.o_proj,
+            )
         qf = ops.head_matmul_rope(
             q, self.uk_t, s.heads, s.rot_dim, positions, self.inv_freq,
             torch.float32,
         )
-        gate = proj[:, s.q_rank + self.kv_cols :] if s.gate else None
         o_lat = ops.ctx_attention_f32(
             qf, cache.k, cache.k[..., : s.kv_rank], meta.block_tables,
             meta.cu_seqlens, meta.context_lens, s.scale, meta.max_seqlen,
@@ -483,6 +497,52 @@ class LatentAttention(nn.Module):
         )
         o = ops.head_matmul_rope(o_lat, self.uv, s.heads)
         return F.linear(o, self.o_proj)
+
+    def _expanded_attention(self, q, gate, positions, cache: LayerCache, meta):
+        """Per-head keys and values of every sequence's whole context, built
+        from its cached rows into scratch pages (numbered 0.. in sequence
+        order), then plain multi-head attention. -> [T, heads * vdim]."""
+        from kserve_amd.ops.torch_ref import rotate_pairs
+
+        s = self.spec
+        H, R, rd = s.heads, s.kv_rank, s.rot_dim
+        T = q.shape[0]
+        q3 = q.view(T, H, s.dim + rd).float()
+        if rd:
+            q3 = torch.cat(
+                [q3[..., : s.dim], rotate_pairs(q3[..., s.dim :], positions, self.inv_freq)],
+                dim=-1,
+            )
+        qf = q3.reshape(T, H * (s.dim + rd)).contiguous()
+        n_seq = meta.cu_seqlens.numel() - 1
+        ctx = meta.context_lens[:n_seq].tolist()  # host read
+        bs = cache.k.shape[2]
+        nbs = [-(-c // bs) for c in ctx]
+        ids = torch.cat(
+            [meta.block_tables[i, :nb] for i, nb in enumerate(nbs)]
+        ).long()
+        rows = cache.k[ids, 0]                       # [pages, bs, R + rd]
+        n_pages = rows.shape[0]
+        lat = rows[..., :R].reshape(-1, R)
+        keys = torch.matmul(lat, self.uk_t)                                  # [H, n, dim]
+        if rd:
+            shared = rows[..., R:].reshape(1, -1, rd).expand(H, -1, -1)
+            keys = torch.cat([keys, shared], dim=-1)
+        vals = torch.matmul(lat, self.uv.transpose(1, 2))                    # [H, n, vdim]
+        k_tmp = keys.view(H, n_pages, bs, -1).transpose(0, 1).contiguous()
+        v_tmp = vals.view(H, n_pages, bs, -1).transpose(0, 1).contiguous()
+        tables = torch.zeros(
+            (n_seq, max(nbs)), dtype=torch.int32, device=q.device
+        )
+        at = 0
+        for i, nb in enumerate(nbs):
+            tables[i, :nb] = torch.arange(at, at + nb, dtype=torch.int32, device=q.device)
+            at += nb
+        return ops.ctx_attention_f32(
+            qf, k_tmp, v_tmp, tables, meta.cu_seqlens, meta.context_lens,
+            s.scale, meta.max_seqlen, H, gate=gate, out_dtype=self.dtype,
+            sink=self.sink, window=s.window,
+        )
 
 
 class GeluMLP(nn.Module):

@@ -115,6 +115,9 @@ class VoboraxForCausalLM(nn.Module):
             if isinstance(l.mlp, SoftmaxRoutedMoE)
         ]
         self.decode_graph_max_tokens = min(caps) if caps else None
+        if any(l.attn.expanded for l in self.layers):
+            # the expanded form of wide rows reads context lengths on the host
+            self.decode_graph_max_tokens = 0
         # when a list, forward() appends the residual stream after each layer
         self.debug_residuals: Optional[List[torch.Tensor]] = None
         self.to(device)

@@ -221,6 +221,34 @@ class TestWholePrompts:
         got = run_schedule(eng, [toks], [[(0, 12)]] + [[(0, 1)]] * 9)[0]
         assert agrees(got, oracle(cfg, sd, toks), backend)
 
+    def test_rows_wider_than_the_kernel_takes(self, backend):
+        """Cached rows of more than 256 columns: keys and values are expanded
+        per head for every step (no captured graphs); portions, decode and
+        two requests side by side in a pool that is used again."""
+        cfg = O.make_config(
+            vocab=40, width=32,
+            layers=[
+                O.windowed(heads=3, dim=8, vdim=12, kv_rank=264, q_rank=16,
+                           rot_dim=8, window=9, mlp=None),
+                O.windowed(heads=2, dim=16, vdim=8, kv_rank=264, q_rank=12,
+                           rot_dim=8, window=30, kv_from=0, mlp=O.dense_cfg(16)),
+                O.sinked(heads=2, dim=8, vdim=8, kv_rank=300, q_rank=16, mlp=None),
+            ],
+        )
+        sd = weights_for(cfg, backend, seed=2)
+        eng = make_engine(cfg, sd, backend, num_blocks=9)
+        assert eng.model.layers[0].attn.expanded
+        assert eng.model.decode_graph_max_tokens == 0
+        prompts = [random_prompt(n, cfg["vocab"], 3 + n) for n in (60, 37, 50)]
+        sched = (
+            [[(0, 17), (1, 5)], [(0, 2), (1, 30)], [(0, 20), (1, 1)], [(1, 1), (0, 1)]]
+            + [[(0, 1)]] * 20 + [[(2, 33)], [(2, 2)]] + [[(2, 1)]] * 15
+        )
+        got = run_schedule(eng, prompts, sched)
+        for i, toks in enumerate(prompts):
+            assert rel_err(got[i], oracle(cfg, sd, toks)) < tol(backend), i
+        assert eng.scheduler.block_manager.num_free_blocks == 8
+
     def test_many_experts_take_the_sorted_path(self, backend):
         """More tokens than the small-batch expert path takes, more router
         outputs than a wave has lanes; some experts get no token at all."""
