@@ -210,14 +210,15 @@ class LLMEngine:
 
                 cap = MixtralMoE.DENSE_MAX_TOKENS
             if cap is not None:
-                self.runner.capture_decode_graphs(
-                    batch_sizes=[
-                        b
-                        for b in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128,
-                                  192, 256, 384)
-                        if b <= cap
-                    ]
-                )
+                buckets = [
+                    b
+                    for b in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128,
+                              192, 256, 384)
+                    if b <= cap
+                ]
+                # a cap below the smallest bucket: every decode step is eager
+                if buckets:
+                    self.runner.capture_decode_graphs(batch_sizes=buckets)
             else:
                 self.runner.capture_decode_graphs()
         logger.info(
