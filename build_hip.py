@@ -46,6 +46,7 @@ MODULES = {
         "sources": [
             "residual_norm_f32.hip",
             "ssm_scan.hip",
+            "linear_scan.hip",
             "attention_f32.hip",
             "latent_attention.hip",
             "moe_route.hip",

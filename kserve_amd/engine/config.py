@@ -187,12 +187,19 @@ class AttentionMixerSpec:
     # chunk-local causal mask: a query sees only keys of its own block of
     # ``chunk`` positions (counted from position 0); 0 = plain causal
     chunk: int = 0
+    # sliding window: a query sees itself and the window-1 positions before
+    # it; 0 = no window
+    window: int = 0
 
     @classmethod
-    def from_dict(cls, d: dict) -> "AttentionMixerSpec":
+    def from_dict(cls, d: dict, mask: str = "chunk") -> "AttentionMixerSpec":
+        """``mask`` says what the entry's ``mask.size`` means in the design
+        that is being read: "chunk" or "window"."""
         qt = d.get("q_temp") or {}
         rot = d.get("rot") or {}
-        mask = d.get("mask") or {}
+        size = int((d.get("mask") or {}).get("size", 0))
+        chunk = size if mask == "chunk" else 0
+        window = size if mask == "window" else 0
         return cls(
             heads=int(d["heads"]),
             kv_heads=int(d.get("kv_heads", d["heads"])),
@@ -203,7 +210,95 @@ class AttentionMixerSpec:
             q_temp_every=int(qt.get("every", 0)),
             rot_dims=int(rot.get("dims", 0)),
             rot_base=float(rot.get("base", 10000.0)),
-            chunk=int(mask.get("size", 0)),
+            chunk=chunk,
+            window=window,
+        )
+
+
+@dataclass
+class RetentionMixerSpec:
+    """Linear attention with a constant decay per head and no softmax:
+    S <- decay_h S + k v^T, o = S^T q, rotary positions on q and k, keys
+    scaled by dim^-1/2, head outputs RMS-normed (no weight) and gated."""
+
+    heads: int
+    dim: int
+    vdim: int
+    decay: list
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "RetentionMixerSpec":
+        rot = d.get("rot") or {}
+        decay = [float(x) for x in d["decay"]]
+        if len(decay) != int(d["heads"]):
+            raise ValueError("one decay per head")
+        return cls(
+            heads=int(d["heads"]),
+            dim=int(d["dim"]),
+            vdim=int(d.get("vdim", d["dim"])),
+            decay=decay,
+            rot_dims=int(rot.get("dims", 0)),
+            rot_base=float(rot.get("base", 10000.0)),
+        )
+
+
+@dataclass
+class DeltaMixerSpec:
+    """Gated delta rule: ``heads`` value heads of ``vdim`` columns, ``kv_heads``
+    query/key heads of ``dim`` columns shared by groups of value heads, a
+    causal convolution of ``conv`` taps + silu on q, k and v, unit-norm q/k, a
+    data-dependent decay and write strength per head."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int = 4
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "DeltaMixerSpec":
+        heads = int(d["heads"])
+        kv = int(d.get("kv_heads", heads))
+        if kv < 1 or heads % kv:
+            raise ValueError("heads must be a multiple of kv_heads")
+        return cls(
+            heads=heads,
+            kv_heads=kv,
+            dim=int(d["dim"]),
+            vdim=int(d.get("vdim", d["dim"])),
+            conv=int(d.get("conv", 4)),
+        )
+
+
+@dataclass
+class SquaredReluMoESpec:
+    """Mixture of two-matrix experts down(relu(up h)^2) routed by sigmoid
+    scores: the ``top`` largest are chosen, their scores are divided by their
+    sum and multiplied by ``scale``, and the weight multiplies the expert's
+    OUTPUT."""
+
+    experts: int
+    top: int
+    ff: int
+    scale: float = 1.0
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "SquaredReluMoESpec":
+        kind = d.get("kind", "moe")
+        if kind != "moe":
+            raise ValueError(f"unsupported feed-forward kind {kind!r}")
+        r = d["router"]
+        return cls(
+            experts=int(r["experts"]),
+            top=int(r["top"]),
+            ff=int(d["expert"]["ff"]),
+            scale=float(r.get("scale", 1.0)),
         )
 
 
@@ -401,6 +496,24 @@ def feed_forward_spec(d: Optional[dict]):
     return GLUSpec.from_dict(d)
 
 
+def laperax_layer_spec(kind: str, mixer: dict, mlp: Optional[dict]):
+    """One Laperax layer: a retention, windowed-attention or delta mixer and
+    an optional mixture of squared-relu experts, both reading one norm."""
+    ff = SquaredReluMoESpec.from_dict(mlp) if mlp else None
+    if kind == "retention":
+        return HybridLayerSpec(
+            kind, retention=RetentionMixerSpec.from_dict(mixer), mlp=ff
+        )
+    if kind == "attention":
+        return HybridLayerSpec(
+            kind, attention=AttentionMixerSpec.from_dict(mixer, mask="window"),
+            mlp=ff,
+        )
+    if kind == "delta":
+        return HybridLayerSpec(kind, delta=DeltaMixerSpec.from_dict(mixer), mlp=ff)
+    raise ValueError(f"unknown layer type {kind!r}")
+
+
 @dataclass
 class LoopSpec:
     """Layers ``start .. stop-1`` run ``times`` times in a row with the same
@@ -421,9 +534,12 @@ class HybridLayerSpec:
     attention: Optional[AttentionMixerSpec] = None
     ssm: Optional[SSMMixerSpec] = None
     latent: Optional[LatentAttentionSpec] = None
+    retention: Optional[RetentionMixerSpec] = None
+    delta: Optional[DeltaMixerSpec] = None
     attention_scale: float = 1.0
     ssm_scale: float = 1.0
-    mlp: Optional[object] = None  # GLUSpec, MoESpec, MLPSpec or SoftmaxMoESpec
+    # GLUSpec, MoESpec, MLPSpec, SoftmaxMoESpec or SquaredReluMoESpec
+    mlp: Optional[object] = None
 
 
 @dataclass
@@ -445,6 +561,9 @@ class HybridModelConfig:
     loop: Optional[LoopSpec] = None
     # every sublayer output is multiplied by this before it joins the stream
     residual_mult: float = 1.0
+    # logits = head x * logit_scale, then cap * tanh(logits / cap) (0: none)
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0
 
     @property
     def num_layers(self) -> int:
@@ -465,7 +584,10 @@ class HybridModelConfig:
 
     @property
     def has_recurrent_state(self) -> bool:
-        return any(l.ssm is not None for l in self.layers)
+        return any(
+            l.ssm is not None or l.retention is not None or l.delta is not None
+            for l in self.layers
+        )
 
     def kv_bytes_per_block(self, block_size: int, itemsize: int) -> int:
         per_token = 0
@@ -481,9 +603,13 @@ class HybridModelConfig:
     @classmethod
     def from_dict(cls, cfg: dict, model_name: str = "merulorn") -> "HybridModelConfig":
         layers = []
+        arch = cfg.get("architecture", "Merulorn")
         for entry in cfg["layers"]:
             kind = entry["type"]
             mixer = entry["mixer"]
+            if arch == "Laperax":
+                layers.append(laperax_layer_spec(kind, mixer, entry.get("mlp")))
+                continue
             if kind in ("latent_attention", "latent_attention_2"):
                 # rotated key part + window + output gate, or none of them
                 # and a sink
@@ -531,6 +657,8 @@ class HybridModelConfig:
             model_name=model_name,
             architecture=cfg.get("architecture", "Merulorn"),
             residual_mult=float(cfg.get("residual_mult", 1.0)),
+            logit_scale=float(cfg.get("logit_scale", 1.0)),
+            logit_softcap=float(cfg.get("logit_softcap", 0.0)),
             loop=(
                 LoopSpec(
                     start=int(cfg["loop"].get("start", 0)),

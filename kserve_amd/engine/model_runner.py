@@ -159,12 +159,16 @@ class ModelRunner:
                 if dv:  # dv 0: the values are columns of the key rows
                     v = alloc((num_blocks, g, bs, dv), dtype=dtype, device=self.device)
                     kv_bytes += v.numel() * v.itemsize
-            if state:
+            # a recurrent layer keeps a convolution history, a matrix state
+            # or both
+            if state.get("conv"):
                 shape, dt = state["conv"]
                 conv = alloc((slots, *shape), dtype=dt, device=self.device)
+                state_bytes += conv.numel() * conv.itemsize
+            if state.get("ssm"):
                 shape, dt = state["ssm"]
                 ssm = alloc((slots, *shape), dtype=dt, device=self.device)
-                state_bytes += conv.numel() * conv.itemsize + ssm.numel() * ssm.itemsize
+                state_bytes += ssm.numel() * ssm.itemsize
             caches.append(LayerCache(k, v, conv, ssm))
         self.kv_caches = caches
         self.num_gpu_blocks = num_blocks

@@ -23,11 +23,14 @@ import torch.nn.functional as F
 from kserve_amd import ops
 from kserve_amd.engine.config import (
     AttentionMixerSpec,
+    DeltaMixerSpec,
     GLUSpec,
     LatentAttentionSpec,
     MLPSpec,
     MoESpec,
+    RetentionMixerSpec,
     SoftmaxMoESpec,
+    SquaredReluMoESpec,
     SSMMixerSpec,
 )
 from kserve_amd.ops.torch_ref import rotary_inv_freq
@@ -40,7 +43,9 @@ class LayerCache(NamedTuple):
     v: Optional[torch.Tensor] = None      # [blocks, kv_heads, block, vdim];
     #                                       None where values are read from k
     conv: Optional[torch.Tensor] = None   # [slots, taps-1, channels]
-    ssm: Optional[torch.Tensor] = None    # [slots, heads, vdim, state] fp32
+    # matrix state of a recurrent layer, fp32: [slots, heads, vdim, state]
+    # (state-space scan) or [slots, heads, vdim, dim] (linear attention)
+    ssm: Optional[torch.Tensor] = None
 
 
 def _param(*shape, dtype):
@@ -173,13 +178,15 @@ class RotaryChunkSinkAttention(nn.Module):
     sink term in the softmax denominator (``sink``), and unit-norm values
     that are rotated by their own position over all of ``vdim`` before they
     are cached, with every head output turned back by the query's position
-    (``value_unit_norm`` / ``rotate_values``). No biases, no gate. The
-    q|k|v projections are one fused GEMM."""
+    (``value_unit_norm`` / ``rotate_values``). ``spec.window`` adds a sliding
+    window. With ``norm_weights`` off the q/k norm has no weights (it then
+    commutes with the rotation, so "rotate, then norm" is the same sublayer).
+    No biases, no gate. The q|k|v projections are one fused GEMM."""
 
     def __init__(
         self, width: int, spec: AttentionMixerSpec, eps: float, dtype,
         sink: bool = True, value_unit_norm: bool = True,
-        rotate_values: bool = True,
+        rotate_values: bool = True, norm_weights: bool = True,
     ):
         super().__init__()
         self.spec = spec
@@ -193,8 +200,8 @@ class RotaryChunkSinkAttention(nn.Module):
         if rotate_values and spec.vdim % 2:
             raise ValueError("rotated values need an even value size")
         self.qkv = _param(self.q_w + self.k_w + self.v_w, width, dtype=dtype)
-        self.q_norm = _param(spec.dim, dtype=torch.float32)
-        self.k_norm = _param(spec.dim, dtype=torch.float32)
+        self.q_norm = _param(spec.dim, dtype=torch.float32) if norm_weights else None
+        self.k_norm = _param(spec.dim, dtype=torch.float32) if norm_weights else None
         self.sink = _param(spec.heads, dtype=torch.float32) if sink else None
         self.o_proj = _param(width, spec.heads * spec.vdim, dtype=dtype)
         self.value_unit_norm = value_unit_norm
@@ -214,8 +221,9 @@ class RotaryChunkSinkAttention(nn.Module):
         self.qkv.copy_(
             torch.cat([get(prefix + n).to(dt) for n in ("q", "k", "v")], dim=0)
         )
-        self.q_norm.copy_(get(prefix + "q.norm").float())
-        self.k_norm.copy_(get(prefix + "k.norm").float())
+        if self.q_norm is not None:
+            self.q_norm.copy_(get(prefix + "q.norm").float())
+            self.k_norm.copy_(get(prefix + "k.norm").float())
         if self.sink is not None:
             self.sink.copy_(get(prefix + "sink").float())
         self.o_proj.copy_(get(prefix + "o").to(dt))
@@ -233,7 +241,7 @@ class RotaryChunkSinkAttention(nn.Module):
             qn, cache.k, cache.v, meta.block_tables, meta.cu_seqlens,
             meta.context_lens, s.scale, meta.max_seqlen, s.heads,
             out_dtype=self.dtype, sink=self.sink, chunk=s.chunk,
-            out_inv_freq=self.v_inv_freq,
+            out_inv_freq=self.v_inv_freq, window=s.window,
         )
         return F.linear(o, self.o_proj)
 
@@ -693,6 +701,234 @@ class SoftmaxRoutedMoE(nn.Module):
             h, self.router, self.spec.top, softmax=True, renorm=True,
             dense=dense, correction=self.correction,
             renorm_eps=self.RENORM_EPS,
+        )
+        if dense:
+            return self._dense(h, dense_w, extra)
+        return self._sorted(h, idx, w, extra)
+
+
+class RetentionMixer(nn.Module):
+    """Linear attention with a constant decay per head (no softmax, no
+    denominator): q, k rotated by their position, k scaled by dim^-1/2, the
+    fp32 state S <- decay_h S + k v^T read out as S^T q, every head output
+    divided by its RMS (no weight), gated by silu of a projection of the
+    sublayer input, out-projection. q|k|v|gate are one fused GEMM."""
+
+    def __init__(self, width: int, spec: RetentionMixerSpec, eps: float, dtype):
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        self.dtype = dtype
+        s = spec
+        if s.rot_dims % 2 or s.rot_dims > s.dim:
+            raise ValueError("rot dims must be even and at most the head size")
+        self.qk_w = s.heads * s.dim
+        self.v_w = s.heads * s.vdim
+        self.qkvg = _param(2 * self.qk_w + 2 * self.v_w, width, dtype=dtype)
+        self.o_proj = _param(width, self.v_w, dtype=dtype)
+        self.register_buffer(
+            "decay", torch.tensor(s.decay, dtype=torch.float32), persistent=False
+        )
+        self.register_buffer(
+            "inv_freq",
+            rotary_inv_freq(s.rot_dims, s.rot_base) if s.rot_dims else None,
+            persistent=False,
+        )
+
+    def state_shapes(self):
+        s = self.spec
+        return {"ssm": ((s.heads, s.vdim, s.dim), torch.float32)}
+
+    def load(self, get, prefix: str):
+        dt = self.dtype
+        self.qkvg.copy_(
+            torch.cat([get(prefix + n).to(dt) for n in ("q", "k", "v", "g")], dim=0)
+        )
+        self.o_proj.copy_(get(prefix + "o").to(dt))
+
+    def forward(self, h, positions, cache: LayerCache, meta):
+        s = self.spec
+        proj = F.linear(h, self.qkvg)
+        a, b, c = self.qk_w, 2 * self.qk_w, 2 * self.qk_w + self.v_w
+        # q | k | v to fp32 in one pass: q and k rotated, k scaled
+        qkv = ops.rope_scale_heads(
+            proj[:, :c], positions, self.inv_freq, s.heads, 1.0, s.heads,
+            s.dim ** -0.5, s.dim,
+        )
+        o = ops.linear_scan(
+            qkv[:, :a], qkv[:, a:b], qkv[:, b:], cache.ssm, positions,
+            meta.cu_seqlens, meta.state_slots, s.heads, decay=self.decay,
+        )
+        on = ops.gated_group_rms_norm(
+            o, proj[:, c:], None, self.eps, s.heads, self.dtype, gate_after=True
+        )
+        return F.linear(on, self.o_proj)
+
+
+class GatedDeltaMixer(nn.Module):
+    """Gated delta rule: q, k, v go through a short causal convolution + silu
+    (history kept per sequence), q and k become unit vectors per head (q also
+    times dim^-1/2), and per value head the fp32 state is decayed by
+    g = exp(-exp(A_log) softplus(a + dt_bias)), corrected towards the value
+    with strength sigmoid(b), S <- S + k (b (v - S^T k))^T, and read as S^T q.
+    Head outputs are RMS-normed with one weight vector shared by the heads,
+    gated by silu of a projection of the input, then out-projected.
+    q|k|v|gate|b|a are one fused GEMM."""
+
+    UNIT_EPS = 1e-6
+
+    def __init__(self, width: int, spec: DeltaMixerSpec, eps: float, dtype):
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        self.dtype = dtype
+        s = spec
+        self.qk_w = s.kv_heads * s.dim
+        self.v_w = s.heads * s.vdim
+        self.proj = _param(
+            s.conv_channels + self.v_w + 2 * s.heads, width, dtype=dtype
+        )
+        self.conv_w = _param(s.conv_channels, s.conv, dtype=torch.float32)
+        self.a_log = _param(s.heads, dtype=torch.float32)
+        self.dt_bias = _param(s.heads, dtype=torch.float32)
+        self.norm_w = _param(s.vdim, dtype=torch.float32)
+        self.o_proj = _param(width, self.v_w, dtype=dtype)
+
+    def state_shapes(self):
+        s = self.spec
+        out = {"ssm": ((s.heads, s.vdim, s.dim), torch.float32)}
+        if s.conv > 1:
+            out["conv"] = ((s.conv - 1, s.conv_channels), self.dtype)
+        return out
+
+    def load(self, get, prefix: str):
+        dt = self.dtype
+        self.proj.copy_(
+            torch.cat(
+                [get(prefix + n).to(dt) for n in ("q", "k", "v", "g", "b", "a")],
+                dim=0,
+            )
+        )
+        self.conv_w.copy_(
+            torch.cat([get(prefix + n + ".conv").float() for n in ("q", "k", "v")], dim=0)
+        )
+        self.a_log.copy_(get(prefix + "A_log").float())
+        self.dt_bias.copy_(get(prefix + "dt_bias").float())
+        self.norm_w.copy_(get(prefix + "norm").float())
+        self.o_proj.copy_(get(prefix + "o").to(dt))
+
+    def forward(self, h, positions, cache: LayerCache, meta):
+        s = self.spec
+        proj = F.linear(h, self.proj)
+        cc = s.conv_channels
+        gate = proj[:, cc : cc + self.v_w]
+        b_raw = proj[:, cc + self.v_w : cc + self.v_w + s.heads]
+        a_raw = proj[:, cc + self.v_w + s.heads :]
+        if s.conv > 1:
+            qkv = ops.causal_conv_silu(
+                proj[:, :cc], self.conv_w, None, cache.conv, positions,
+                meta.seq_of_token, meta.cu_seqlens, meta.state_slots,
+            )
+        else:
+            x = proj[:, :cc].float() * self.conv_w[:, 0]
+            qkv = x * torch.sigmoid(x)
+        ops.unit_norm_heads(
+            qkv, s.kv_heads, s.dim ** -0.5, s.kv_heads, 1.0, s.dim, self.UNIT_EPS
+        )
+        a = self.qk_w
+        o = ops.linear_scan(
+            qkv[:, :a], qkv[:, a : 2 * a], qkv[:, 2 * a :], cache.ssm, positions,
+            meta.cu_seqlens, meta.state_slots, s.kv_heads, a_raw=a_raw,
+            b_raw=b_raw, a_log=self.a_log, dt_bias=self.dt_bias,
+        )
+        on = ops.gated_group_rms_norm(
+            o, gate, self.norm_w, self.eps, s.heads, self.dtype, gate_after=True
+        )
+        return F.linear(on, self.o_proj)
+
+
+class SquaredReluMoE(nn.Module):
+    """Mixture of two-matrix experts down(relu(up h)^2) without biases. fp32
+    router logits, sigmoid scores, the ``top`` largest chosen and weighted by
+    score / (sum of the chosen scores + 1e-20) * scale; the weight multiplies
+    the expert's OUTPUT; the weighted sum is fp32, and ``extra`` (another
+    sublayer's output for the same tokens) joins that sum.
+
+    Weights: up stacked as [E, ff, width] (also one [E * ff, width] matrix),
+    down as [width, E, ff] (also one [width, E * ff] matrix). Small batches
+    and captured decode graphs run every expert on every token: ONE GEMM
+    against all up rows, the activation scaled by the token's weight for that
+    expert (zero where it was not chosen), ONE GEMM against all down columns,
+    which sums over the experts in its fp32 accumulator. Larger batches sort
+    the (token, expert) pairs by expert and run a GEMM pair per expert on its
+    contiguous rows."""
+
+    DENSE_ROW_BUDGET = RoutedClampedMoE.DENSE_ROW_BUDGET
+    RENORM_EPS = 1e-20
+
+    def __init__(self, width: int, spec: SquaredReluMoESpec, dtype):
+        super().__init__()
+        self.spec = spec
+        self.dtype = dtype
+        E = spec.experts
+        if not 1 <= spec.top <= E:
+            raise ValueError("top must be between 1 and the number of experts")
+        self.dense_max_tokens = max(16, self.DENSE_ROW_BUDGET * spec.top // E)
+        self.router = _param(E, width, dtype=torch.float32)
+        self.up = _param(E, spec.ff, width, dtype=dtype)
+        self.down = _param(width, E, spec.ff, dtype=dtype)
+
+    def load(self, get, prefix: str):
+        dt = self.dtype
+        self.router.copy_(get(prefix + "router").float())
+        for e in range(self.spec.experts):
+            p = f"{prefix}e{e}."
+            self.up[e].copy_(get(p + "up").to(dt))
+            self.down[:, e].copy_(get(p + "down").to(dt))
+
+    def _dense(self, h, dense_w, extra):
+        E, ff = self.spec.experts, self.spec.ff
+        T, W = h.shape
+        x = F.linear(h, self.up.view(E * ff, W))
+        act = ops.relu2_scale(x.view(T * E, ff), dense_w.reshape(-1))
+        y = F.linear(act.view(T, E * ff), self.down.view(W, E * ff))
+        ar = torch.arange(T, dtype=torch.int32, device=h.device)
+        return ops.combine_rows(y, ar, 1, extra)
+
+    def _sorted(self, h, idx, w, extra):
+        E, top = self.spec.experts, self.spec.top
+        flat = idx.view(-1).long()
+        order = torch.sort(flat, stable=True).indices
+        counts = torch.bincount(flat, minlength=E).tolist()  # host sync
+        xs = ops.gather_scale_rows(h, (order // top).to(torch.int32))
+        n = xs.shape[0]
+        x = torch.empty((n, self.spec.ff), dtype=h.dtype, device=h.device)
+        a = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.mm(xs[a : a + c], self.up[e].t(), out=x[a : a + c])
+            a += c
+        act = ops.relu2_scale(x)
+        ys = torch.empty_like(xs)
+        a = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.mm(act[a : a + c], self.down[:, e].t(), out=ys[a : a + c])
+            a += c
+        # pair p = t*top + k sits at sorted row inv[p]
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(n, device=h.device)
+        return ops.combine_rows(ys, inv.to(torch.int32), top, extra, w.view(-1))
+
+    def forward(self, h, extra=None):
+        """[T, width] in the activation dtype -> fp32 [T, width]."""
+        T = h.shape[0]
+        dense = T <= self.dense_max_tokens or (
+            h.is_cuda and torch.cuda.is_current_stream_capturing()
+        )
+        idx, w, dense_w, _ = ops.route_tokens(
+            h, self.router, self.spec.top, renorm=True, dense=dense,
+            renorm_eps=self.RENORM_EPS, weight_scale=self.spec.scale,
         )
         if dense:
             return self._dense(h, dense_w, extra)

@@ -56,6 +56,12 @@ register(
     "kserve_amd.models.voborax.VoboraxForCausalLM",
     ("kserve_amd_seq_C",),
 )
+register(
+    "Laperax",
+    "kserve_amd.engine.config.HybridModelConfig",
+    "kserve_amd.models.laperax.LaperaxForCausalLM",
+    ("kserve_amd_seq_C",),
+)
 
 
 def architecture_of(config_json: dict) -> str:

@@ -362,14 +362,22 @@ def add_rms_norm_f32res(
     )
 
 
-def gated_group_rms_norm(y, z, weight, eps: float, groups: int, out_dtype):
+def gated_group_rms_norm(
+    y, z, weight, eps: float, groups: int, out_dtype, gate_after: bool = False
+):
+    """RMS norm of fp32 ``y`` in ``groups`` equal parts with a silu(z) gate:
+    on the input of the norm, or (``gate_after``) on its output. ``weight``
+    may be shorter than a row (it repeats: one vector shared by the groups)
+    or None."""
     if y.is_cuda:
         out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
         _native_seq("gated_group_rms_norm").gated_group_rms_norm(
-            out, y, z, weight, float(eps), int(groups)
+            out, y, z, weight, float(eps), int(groups), bool(gate_after)
         )
         return out
-    return torch_ref.gated_group_rms_norm(y, z, weight, eps, groups, out_dtype)
+    return torch_ref.gated_group_rms_norm(
+        y, z, weight, eps, groups, out_dtype, gate_after
+    )
 
 
 def causal_conv_silu(
@@ -502,6 +510,7 @@ def post_norm_add_rms_norm(
 def router_topk(
     logits, top: int, softmax: bool = False, renorm: bool = False,
     dense: bool = False, correction=None, renorm_eps: float = 0.0,
+    weight_scale: float = 1.0,
 ):
     """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32
     [T, top], dense [T, E] weights or None) by sigmoid (or softmax) score;
@@ -516,18 +525,19 @@ def router_topk(
         )
         _native_seq("router_topk").router_topk(
             idx, w, dw, logits, bool(softmax), bool(renorm), correction,
-            float(renorm_eps),
+            float(renorm_eps), float(weight_scale),
         )
         return idx, w, dw
     return torch_ref.router_topk(
-        logits, top, softmax, renorm, dense, correction, renorm_eps
+        logits, top, softmax, renorm, dense, correction, renorm_eps,
+        weight_scale,
     )
 
 
 def route_tokens(
     h, router, top: int, softmax: bool = False, renorm: bool = False,
     dense: bool = False, want_logits: bool = False, correction=None,
-    renorm_eps: float = 0.0,
+    renorm_eps: float = 0.0, weight_scale: float = 1.0,
 ):
     """The router in one kernel: fp32 logits of h [T, W] (activation dtype)
     against fp32 router rows [E, W], scores, the ``top`` experts. Returns
@@ -542,12 +552,12 @@ def route_tokens(
         lg = torch.empty((T, E), dtype=torch.float32, device=dev) if want_logits else None
         _native_seq("route_tokens").route_tokens(
             idx, w, dw, lg, h, router, bool(softmax), bool(renorm), correction,
-            float(renorm_eps),
+            float(renorm_eps), float(weight_scale),
         )
         return idx, w, dw, lg
     return torch_ref.route_tokens(
         h, router, top, softmax, renorm, dense, want_logits, correction,
-        renorm_eps,
+        renorm_eps, weight_scale,
     )
 
 
@@ -671,3 +681,83 @@ def bias_gelu_tanh(x, bias):
         _native_seq("bias_gelu_tanh").bias_gelu_tanh(out, x, bias)
         return out
     return torch_ref.bias_gelu_tanh(x, bias)
+
+
+# -- linear-attention recurrences, squared-relu experts, capped logits --------
+
+def rope_scale_heads(
+    x, positions, inv_freq, heads_a: int, scale_a: float, heads_b: int,
+    scale_b: float, dim: int,
+):
+    """fp32 copy of rows x [T, width]: the first ``heads_a`` heads of ``dim``
+    columns get rotary positions on their first 2*len(inv_freq) coordinates
+    (i pairs with i + half) and are multiplied by scale_a, the next
+    ``heads_b`` likewise with scale_b; further columns are only widened."""
+    if x.is_cuda:
+        out = _f32_like(x.shape[0], x.shape[1], x)
+        _native_seq("rope_scale_heads").rope_scale_heads(
+            out, x, positions, inv_freq, int(heads_a), float(scale_a),
+            int(heads_b), float(scale_b), int(dim),
+        )
+        return out
+    return torch_ref.rope_scale_heads(
+        x, positions, inv_freq, heads_a, scale_a, heads_b, scale_b, dim
+    )
+
+
+def unit_norm_heads(
+    x, heads_a: int, scale_a: float, heads_b: int, scale_b: float, dim: int,
+    eps: float,
+):
+    """In place on fp32 rows: the first ``heads_a`` heads of ``dim`` columns
+    become x / sqrt(sum(x^2) + eps) * scale_a, the next ``heads_b`` likewise
+    with scale_b; further columns are left alone."""
+    if x.is_cuda:
+        _native_seq("unit_norm_heads").unit_norm_heads(
+            x, int(heads_a), float(scale_a), int(heads_b), float(scale_b),
+            int(dim), float(eps),
+        )
+        return x
+    return torch_ref.unit_norm_heads(x, heads_a, scale_a, heads_b, scale_b, dim, eps)
+
+
+def linear_scan(
+    q, k, v, state, positions, cu_seqlens, slots, qk_heads: int,
+    decay=None, a_raw=None, b_raw=None, a_log=None, dt_bias=None,
+):
+    """Linear-attention recurrence over a flat varlen batch; carries
+    ``state[slot]`` ([heads, V, K] fp32). q, k [T, qk_heads*K] and
+    v [T, heads*V] are fp32 (rows may be strided). With ``decay`` [heads]:
+    S <- d S + k v^T. Without: the gated delta rule with
+    g = exp(-exp(a_log) softplus(a_raw + dt_bias)), b = sigmoid(b_raw):
+    S <- g S; S <- S + k (b (v - S^T k))^T. Output o = S^T q, fp32."""
+    if q.is_cuda:
+        heads, V = state.shape[1], state.shape[2]
+        o = _f32_like(q.shape[0], heads * V, q)
+        _native_seq("linear_scan").linear_scan(
+            o, q, k, v, decay, a_raw, b_raw, a_log, dt_bias, state, positions,
+            cu_seqlens, slots, int(qk_heads),
+        )
+        return o
+    return torch_ref.linear_scan(
+        q, k, v, state, positions, cu_seqlens, slots, qk_heads, decay, a_raw,
+        b_raw, a_log, dt_bias,
+    )
+
+
+def relu2_scale(x, scales=None):
+    """max(x, 0)^2 (* scales[row]) in x's dtype."""
+    if x.is_cuda:
+        out = torch.empty_like(x)
+        _native_seq("relu2_scale").relu2_scale(out, x, scales)
+        return out
+    return torch_ref.relu2_scale(x, scales)
+
+
+def scale_softcap(x, scale: float, cap: float):
+    """fp32 cap * tanh(x * scale / cap); cap 0 leaves x * scale."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        _native_seq("scale_softcap").scale_softcap(out, x, float(scale), float(cap))
+        return out
+    return torch_ref.scale_softcap(x, scale, cap)

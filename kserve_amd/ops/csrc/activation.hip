@@ -10,6 +10,8 @@
 // (token, expert) routing weight into the activation this way.
 // bias_gelu_tanh: out = gelu_tanh(x + bias[col]),
 // gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+// relu2_scale: out = max(x, 0)^2 * scale[row] (scale optional), same dtype.
+// scale_softcap: fp32 out = cap * tanh(x * scale / cap) (cap 0: x * scale).
 #include "dtype_io.h"
 
 namespace {
@@ -64,6 +66,63 @@ __global__ void glu_silu_scale_bf16x8_kernel(short* __restrict__ out,
       }
     }
     out_vec[idx] = o;
+  }
+}
+
+template <typename T>
+__global__ void relu2_scale_kernel(T* __restrict__ out,
+                                   const T* __restrict__ input,
+                                   const float* __restrict__ scales,
+                                   const long rows, const int d) {
+  const long total = rows * d;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const float sc = scales ? scales[idx / d] : 1.0f;
+    float y = 0.f;
+    if (!scales || sc != 0.0f) {
+      const float x = fmaxf(ld_f32(input, idx), 0.f);
+      y = x * x * sc;
+    }
+    st_f32(out, idx, y);
+  }
+}
+
+__global__ void relu2_scale_bf16x8_kernel(short* __restrict__ out,
+                                          const short* __restrict__ input,
+                                          const float* __restrict__ scales,
+                                          const long rows, const int d) {
+  const int nvec = d >> 3;
+  const short8_t* in_vec = reinterpret_cast<const short8_t*>(input);
+  short8_t* out_vec = reinterpret_cast<short8_t*>(out);
+  const long total = rows * nvec;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const float sc = scales ? scales[idx / nvec] : 1.0f;
+    short8_t o;
+    if (scales && sc == 0.0f) {
+      // an expert the token did not choose: nothing to read
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = 0;
+    } else {
+      const short8_t x8 = in_vec[idx];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float x = fmaxf(bf16_bits_to_float(x8[j]), 0.f);
+        o[j] = float_to_bf16_bits(x * x * sc);
+      }
+    }
+    out_vec[idx] = o;
+  }
+}
+
+template <typename T>
+__global__ void scale_softcap_kernel(float* __restrict__ out,
+                                     const T* __restrict__ input, float scale,
+                                     float cap, const long total) {
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const float x = ld_f32(input, idx) * scale;
+    out[idx] = cap > 0.f ? cap * tanhf(x / cap) : x;
   }
 }
 
@@ -267,6 +326,51 @@ extern "C" hipError_t ks_bias_gelu_tanh(void* out, const void* input,
     hipLaunchKernelGGL(bias_gelu_tanh_kernel<short>, dim3(grid), dim3(256), 0,
                        stream, (short*)out, (const short*)input,
                        (const float*)bias, (long)rows, d);
+  HIP_CHECK_KERNEL();
+  return hipSuccess;
+}
+
+extern "C" hipError_t ks_relu2_scale(void* out, const void* input,
+                                     const void* scales, int rows, int d,
+                                     int is_f32, hipStream_t stream) {
+  const long total = (long)rows * d;
+  if (total == 0) return hipSuccess;
+  int grid = (int)((total + 255) / 256);
+  if (grid > 4096) grid = 4096;
+  if (is_f32)
+    hipLaunchKernelGGL(relu2_scale_kernel<float>, dim3(grid), dim3(256), 0,
+                       stream, (float*)out, (const float*)input,
+                       (const float*)scales, (long)rows, d);
+  else if (d % 8 == 0 && ((uintptr_t)input % 16) == 0 &&
+           ((uintptr_t)out % 16) == 0) {
+    const long tv = (long)rows * (d >> 3);
+    int gv = (int)((tv + 255) / 256);
+    if (gv > 8192) gv = 8192;
+    hipLaunchKernelGGL(relu2_scale_bf16x8_kernel, dim3(gv), dim3(256), 0,
+                       stream, (short*)out, (const short*)input,
+                       (const float*)scales, (long)rows, d);
+  } else
+    hipLaunchKernelGGL(relu2_scale_kernel<short>, dim3(grid), dim3(256), 0,
+                       stream, (short*)out, (const short*)input,
+                       (const float*)scales, (long)rows, d);
+  HIP_CHECK_KERNEL();
+  return hipSuccess;
+}
+
+extern "C" hipError_t ks_scale_softcap(void* out, const void* input,
+                                       float scale, float cap, long total,
+                                       int is_f32, hipStream_t stream) {
+  if (total == 0) return hipSuccess;
+  int grid = (int)((total + 255) / 256);
+  if (grid > 4096) grid = 4096;
+  if (is_f32)
+    hipLaunchKernelGGL(scale_softcap_kernel<float>, dim3(grid), dim3(256), 0,
+                       stream, (float*)out, (const float*)input, scale, cap,
+                       total);
+  else
+    hipLaunchKernelGGL(scale_softcap_kernel<short>, dim3(grid), dim3(256), 0,
+                       stream, (float*)out, (const short*)input, scale, cap,
+                       total);
   HIP_CHECK_KERNEL();
   return hipSuccess;
 }

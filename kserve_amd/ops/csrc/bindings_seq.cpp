@@ -10,10 +10,10 @@ hipError_t ks_embed_scale_sinpos(void*, const void*, const void*, const void*,
                                  hipStream_t);
 hipError_t ks_add_rms_norm_f32res(void*, const void*, long, float, const void*,
                                   long, float, const void*, float, float,
-                                  void*, int, int, int, hipStream_t);
+                                  void*, int, int, int, int, hipStream_t);
 hipError_t ks_gated_group_rms_norm(void*, const void*, const void*, long,
-                                   const void*, float, int, int, int, int,
-                                   hipStream_t);
+                                   const void*, int, float, int, int, int, int,
+                                   int, hipStream_t);
 hipError_t ks_causal_conv_silu(void*, const void*, long, const void*,
                                const void*, void*, const void*, const void*,
                                const void*, const void*, int, int, int, int,
@@ -45,10 +45,10 @@ hipError_t ks_post_norm_add_rms_norm(void*, const void*, long, int, float,
                                      float, float, void*, int, int, int,
                                      hipStream_t);
 hipError_t ks_router_topk(void*, void*, void*, const void*, int, int, int, int,
-                          int, const void*, float, hipStream_t);
+                          int, const void*, float, float, hipStream_t);
 hipError_t ks_route_tokens(void*, void*, void*, void*, const void*, long,
                            const void*, int, int, int, int, int, int,
-                           const void*, float, int, hipStream_t);
+                           const void*, float, float, int, hipStream_t);
 hipError_t ks_gather_scale_rows(void*, const void*, long, const void*,
                                 const void*, int, int, int, hipStream_t);
 hipError_t ks_combine_rows(void*, const void*, const void*, int, const void*,
@@ -70,6 +70,20 @@ hipError_t ks_bias_gelu_tanh(void*, const void*, const void*, int, int, int,
                              hipStream_t);
 hipError_t ks_clamped_swiglu(void*, const void*, int, int, float, float, int,
                              hipStream_t);
+hipError_t ks_relu2_scale(void*, const void*, const void*, int, int, int,
+                          hipStream_t);
+hipError_t ks_scale_softcap(void*, const void*, float, float, long, int,
+                            hipStream_t);
+hipError_t ks_rope_scale_heads(void*, const void*, long, const void*,
+                               const void*, int, int, int, float, int, float,
+                               int, int, int, hipStream_t);
+hipError_t ks_unit_norm_heads(void*, long, int, int, float, int, float, int,
+                              float, hipStream_t);
+hipError_t ks_linear_scan(void*, const void*, long, const void*, long,
+                          const void*, long, const void*, const void*,
+                          const void*, long, int, const void*, const void*,
+                          void*, const void*, const void*, const void*, int,
+                          int, int, int, int, hipStream_t);
 }
 
 namespace {
@@ -138,11 +152,16 @@ void add_rms_norm_f32res(at::Tensor& residual,
   TORCH_CHECK(weight.numel() == width && out.numel() == residual.numel(),
               "add_rms_norm_f32res: shape mismatch");
   const int f32 = act_is_f32(out, "out");
+  // the deltas share a dtype: the output's, or fp32 beside a bf16 output
+  int df32 = f32;
+  if (d0.has_value()) df32 = act_is_f32(*d0, "d0");
+  else if (d1.has_value()) df32 = act_is_f32(*d1, "d1");
+  TORCH_CHECK(df32 == f32 || df32 == 1, "bf16 deltas need a bf16 output");
   const void *p0 = nullptr, *p1 = nullptr;
   long st0 = 0, st1 = 0;
   if (d0.has_value()) {
     CHECK_ROWS(*d0);
-    TORCH_CHECK(act_is_f32(*d0, "d0") == f32 && d0->size(0) == rows &&
+    TORCH_CHECK(act_is_f32(*d0, "d0") == df32 && d0->size(0) == rows &&
                     d0->size(1) == width,
                 "d0: dtype/shape mismatch");
     p0 = d0->data_ptr();
@@ -150,7 +169,7 @@ void add_rms_norm_f32res(at::Tensor& residual,
   }
   if (d1.has_value()) {
     CHECK_ROWS(*d1);
-    TORCH_CHECK(act_is_f32(*d1, "d1") == f32 && d1->size(0) == rows &&
+    TORCH_CHECK(act_is_f32(*d1, "d1") == df32 && d1->size(0) == rows &&
                     d1->size(1) == width,
                 "d1: dtype/shape mismatch");
     p1 = d1->data_ptr();
@@ -159,37 +178,50 @@ void add_rms_norm_f32res(at::Tensor& residual,
   check_hip(ks_add_rms_norm_f32res(residual.data_ptr(), p0, st0, (float)s0, p1,
                                    st1, (float)s1, weight.data_ptr(),
                                    (float)w_offset, (float)eps, out.data_ptr(),
-                                   rows, width, f32, current_stream()),
+                                   rows, width, f32, df32, current_stream()),
             "add_rms_norm_f32res");
 }
 
 void gated_group_rms_norm(at::Tensor& out, at::Tensor& y, at::Tensor& z,
-                          at::Tensor& weight, double eps, int64_t groups) {
+                          const c10::optional<at::Tensor>& weight_opt,
+                          double eps, int64_t groups, bool gate_after) {
   CHECK_F32(y);
-  CHECK_F32(weight);
+  const void* wp = nullptr;
+  int64_t wn = y.size(1);
+  if (weight_opt.has_value()) {
+    CHECK_F32(*weight_opt);
+    wp = weight_opt->data_ptr();
+    wn = weight_opt->numel();
+  }
   CHECK_ROWS(z);
   TORCH_CHECK(y.dim() == 2 && out.is_contiguous(), "y [T, inner]");
   const int rows = y.size(0), inner = y.size(1);
   const int f32 = act_is_f32(out, "out");
   TORCH_CHECK(act_is_f32(z, "z") == f32 && z.size(0) == rows &&
-                  z.size(1) == inner && weight.numel() == inner &&
+                  z.size(1) == inner && wn > 0 && inner % wn == 0 &&
                   out.numel() == y.numel() && groups > 0 &&
                   inner % groups == 0,
               "gated_group_rms_norm: dtype/shape mismatch");
   check_hip(ks_gated_group_rms_norm(out.data_ptr(), y.data_ptr(), z.data_ptr(),
-                                    z.stride(0), weight.data_ptr(), (float)eps,
-                                    rows, inner, (int)groups, f32,
-                                    current_stream()),
+                                    z.stride(0), wp, (int)wn, (float)eps, rows,
+                                    inner, (int)groups, gate_after ? 1 : 0,
+                                    f32, current_stream()),
             "gated_group_rms_norm");
 }
 
 void causal_conv_silu(at::Tensor& out, at::Tensor& in, at::Tensor& w,
-                      at::Tensor& bias, at::Tensor& conv_state,
+                      const c10::optional<at::Tensor>& bias_opt,
+                      at::Tensor& conv_state,
                       at::Tensor& positions, at::Tensor& seq_of_token,
                       at::Tensor& cu_seqlens, at::Tensor& slots) {
   CHECK_F32(out);
   CHECK_F32(w);
-  CHECK_F32(bias);
+  const void* bias_ptr = nullptr;
+  if (bias_opt.has_value()) {
+    CHECK_F32(*bias_opt);
+    TORCH_CHECK(bias_opt->numel() == in.size(1), "bias [channels]");
+    bias_ptr = bias_opt->data_ptr();
+  }
   CHECK_ROWS(in);
   CHECK_I64(positions);
   CHECK_I32(seq_of_token);
@@ -199,7 +231,6 @@ void causal_conv_silu(at::Tensor& out, at::Tensor& in, at::Tensor& w,
   const int taps = w.size(1), num_seqs = slots.numel();
   const int f32 = act_is_f32(in, "in");
   TORCH_CHECK(w.dim() == 2 && w.size(0) == channels &&
-                  bias.numel() == channels &&
                   out.numel() == (int64_t)tokens * channels &&
                   positions.numel() >= tokens &&
                   seq_of_token.numel() >= tokens &&
@@ -211,7 +242,7 @@ void causal_conv_silu(at::Tensor& out, at::Tensor& in, at::Tensor& w,
                   conv_state.size(2) == channels,
               "conv_state must be [slots, taps-1, channels] in the input dtype");
   check_hip(ks_causal_conv_silu(out.data_ptr(), in.data_ptr(), in.stride(0),
-                                w.data_ptr(), bias.data_ptr(),
+                                w.data_ptr(), bias_ptr,
                                 conv_state.data_ptr(), positions.data_ptr(),
                                 seq_of_token.data_ptr(), cu_seqlens.data_ptr(),
                                 slots.data_ptr(), tokens, num_seqs, channels,
@@ -381,7 +412,9 @@ void ctx_attention_f32(at::Tensor& out, at::Tensor& q, at::Tensor& k_cache,
 }
 
 void qk_headnorm_rope_cache(at::Tensor& q_out, at::Tensor& q, at::Tensor& k,
-                            at::Tensor& v, at::Tensor& qw, at::Tensor& kw,
+                            at::Tensor& v,
+                            const c10::optional<at::Tensor>& qw_opt,
+                            const c10::optional<at::Tensor>& kw_opt,
                             at::Tensor& positions, at::Tensor& slot_mapping,
                             at::Tensor& k_cache, at::Tensor& v_cache,
                             double eps, int64_t heads,
@@ -389,8 +422,18 @@ void qk_headnorm_rope_cache(at::Tensor& q_out, at::Tensor& q, at::Tensor& k,
                             bool v_unit_norm,
                             const c10::optional<at::Tensor>& v_inv_freq) {
   CHECK_F32(q_out);
-  CHECK_F32(qw);
-  CHECK_F32(kw);
+  // without weights the norm is plain x / rms(x)
+  const void *qwp = nullptr, *kwp = nullptr;
+  if (qw_opt.has_value()) {
+    CHECK_F32(*qw_opt);
+    TORCH_CHECK(qw_opt->numel() == k_cache.size(3), "qw [dim]");
+    qwp = qw_opt->data_ptr();
+  }
+  if (kw_opt.has_value()) {
+    CHECK_F32(*kw_opt);
+    TORCH_CHECK(kw_opt->numel() == k_cache.size(3), "kw [dim]");
+    kwp = kw_opt->data_ptr();
+  }
   CHECK_ROWS(q);
   CHECK_ROWS(k);
   CHECK_ROWS(v);
@@ -410,8 +453,7 @@ void qk_headnorm_rope_cache(at::Tensor& q_out, at::Tensor& q, at::Tensor& k,
   TORCH_CHECK(q.size(1) == heads * D && k.size(1) == G * D &&
                   v.size(1) == G * DV && k.size(0) == tokens &&
                   v.size(0) == tokens && q.stride(0) == k.stride(0) &&
-                  q.stride(0) == v.stride(0) && qw.numel() == D &&
-                  kw.numel() == D && v_cache.size(1) == G &&
+                  q.stride(0) == v.stride(0) && v_cache.size(1) == G &&
                   v_cache.size(2) == bs && v_cache.size(0) == k_cache.size(0) &&
                   q_out.numel() == (int64_t)tokens * heads * D &&
                   positions.numel() >= tokens && slot_mapping.numel() >= tokens,
@@ -432,7 +474,7 @@ void qk_headnorm_rope_cache(at::Tensor& q_out, at::Tensor& q, at::Tensor& k,
   }
   check_hip(ks_qk_headnorm_rope_cache(
                 q_out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                q.stride(0), qw.data_ptr(), kw.data_ptr(),
+                q.stride(0), qwp, kwp,
                 positions.data_ptr(), slot_mapping.data_ptr(),
                 k_cache.data_ptr(), v_cache.data_ptr(), (float)eps, tokens,
                 (int)heads, G, D, DV, bs, qf, qh, v_unit_norm ? 1 : 0, vf, vh,
@@ -494,7 +536,7 @@ void router_topk(at::Tensor& idx, at::Tensor& w,
                  const c10::optional<at::Tensor>& dense, at::Tensor& logits,
                  bool softmax, bool renorm,
                  const c10::optional<at::Tensor>& correction,
-                 double renorm_eps) {
+                 double renorm_eps, double weight_scale) {
   CHECK_F32(logits);
   CHECK_F32(w);
   CHECK_I32(idx);
@@ -516,7 +558,8 @@ void router_topk(at::Tensor& idx, at::Tensor& w,
   }
   check_hip(ks_router_topk(idx.data_ptr(), w.data_ptr(), dp, logits.data_ptr(),
                            T, E, top, softmax ? 1 : 0, renorm ? 1 : 0, cp,
-                           (float)renorm_eps, current_stream()),
+                           (float)renorm_eps, (float)weight_scale,
+                           current_stream()),
             "router_topk");
 }
 
@@ -525,7 +568,7 @@ void route_tokens(at::Tensor& idx, at::Tensor& w,
                   const c10::optional<at::Tensor>& logits_out, at::Tensor& h,
                   at::Tensor& router, bool softmax, bool renorm,
                   const c10::optional<at::Tensor>& correction,
-                  double renorm_eps) {
+                  double renorm_eps, double weight_scale) {
   CHECK_ROWS(h);
   CHECK_F32(router);
   CHECK_F32(w);
@@ -556,7 +599,8 @@ void route_tokens(at::Tensor& idx, at::Tensor& w,
   check_hip(ks_route_tokens(idx.data_ptr(), w.data_ptr(), dp, lp, h.data_ptr(),
                             h.stride(0), router.data_ptr(), T, W, E, top,
                             softmax ? 1 : 0, renorm ? 1 : 0, cp,
-                            (float)renorm_eps, act_is_f32(h, "h"),
+                            (float)renorm_eps, (float)weight_scale,
+                            act_is_f32(h, "h"),
                             current_stream()),
             "route_tokens");
 }
@@ -788,6 +832,148 @@ void glu_silu_scale(at::Tensor& out, at::Tensor& input,
             "glu_silu_scale");
 }
 
+void relu2_scale(at::Tensor& out, at::Tensor& input,
+                 const c10::optional<at::Tensor>& scales) {
+  TORCH_CHECK(input.dim() == 2 && input.is_contiguous() && out.is_contiguous(),
+              "input [rows, d] contiguous");
+  const int rows = input.size(0), d = input.size(1);
+  const int f32 = act_is_f32(input, "input");
+  TORCH_CHECK(act_is_f32(out, "out") == f32 && out.numel() == input.numel(),
+              "relu2_scale: dtype/shape mismatch");
+  const void* sp = nullptr;
+  if (scales.has_value()) {
+    CHECK_F32(*scales);
+    TORCH_CHECK(scales->numel() == rows, "scales [rows]");
+    sp = scales->data_ptr();
+  }
+  check_hip(ks_relu2_scale(out.data_ptr(), input.data_ptr(), sp, rows, d, f32,
+                           current_stream()),
+            "relu2_scale");
+}
+
+void scale_softcap(at::Tensor& out, at::Tensor& input, double scale,
+                   double cap) {
+  CHECK_F32(out);
+  TORCH_CHECK(input.is_contiguous() && out.numel() == input.numel(),
+              "scale_softcap: shape mismatch");
+  check_hip(ks_scale_softcap(out.data_ptr(), input.data_ptr(), (float)scale,
+                             (float)cap, (long)input.numel(),
+                             act_is_f32(input, "input"), current_stream()),
+            "scale_softcap");
+}
+
+void rope_scale_heads(at::Tensor& out, at::Tensor& in, at::Tensor& positions,
+                      const c10::optional<at::Tensor>& inv_freq,
+                      int64_t heads_a, double scale_a, int64_t heads_b,
+                      double scale_b, int64_t dim) {
+  CHECK_F32(out);
+  CHECK_ROWS(in);
+  CHECK_I64(positions);
+  const int tokens = in.size(0), width = in.size(1);
+  TORCH_CHECK(heads_a >= 0 && heads_b >= 0 && dim > 0 &&
+                  (heads_a + heads_b) * dim <= width &&
+                  out.numel() == (int64_t)tokens * width &&
+                  positions.numel() >= tokens,
+              "rope_scale_heads: shape mismatch");
+  const void* fp = nullptr;
+  int half = 0;
+  if (inv_freq.has_value()) {
+    CHECK_F32(*inv_freq);
+    half = inv_freq->numel();
+    TORCH_CHECK(2 * half <= dim, "more rotated coordinates than the head has");
+    fp = inv_freq->data_ptr();
+  }
+  check_hip(ks_rope_scale_heads(out.data_ptr(), in.data_ptr(), in.stride(0),
+                                positions.data_ptr(), fp, half, tokens,
+                                (int)heads_a, (float)scale_a, (int)heads_b,
+                                (float)scale_b, (int)dim, width,
+                                act_is_f32(in, "in"), current_stream()),
+            "rope_scale_heads");
+}
+
+void unit_norm_heads(at::Tensor& x, int64_t heads_a, double scale_a,
+                     int64_t heads_b, double scale_b, int64_t dim, double eps) {
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == at::kFloat, "x must be fp32");
+  CHECK_ROWS(x);
+  TORCH_CHECK(heads_a >= 0 && heads_b >= 0 && dim > 0 &&
+                  (heads_a + heads_b) * dim <= x.size(1),
+              "unit_norm_heads: more head columns than the rows have");
+  check_hip(ks_unit_norm_heads(x.data_ptr(), x.stride(0), (int)x.size(0),
+                               (int)heads_a, (float)scale_a, (int)heads_b,
+                               (float)scale_b, (int)dim, (float)eps,
+                               current_stream()),
+            "unit_norm_heads");
+}
+
+void linear_scan(at::Tensor& o, at::Tensor& q, at::Tensor& k, at::Tensor& v,
+                 const c10::optional<at::Tensor>& decay,
+                 const c10::optional<at::Tensor>& a_raw,
+                 const c10::optional<at::Tensor>& b_raw,
+                 const c10::optional<at::Tensor>& a_log,
+                 const c10::optional<at::Tensor>& dt_bias, at::Tensor& state,
+                 at::Tensor& positions, at::Tensor& cu_seqlens,
+                 at::Tensor& slots, int64_t qk_heads) {
+  CHECK_F32(o);
+  CHECK_F32(state);
+  CHECK_ROWS(q);
+  CHECK_ROWS(k);
+  CHECK_ROWS(v);
+  CHECK_I64(positions);
+  CHECK_I32(cu_seqlens);
+  CHECK_I32(slots);
+  TORCH_CHECK(q.scalar_type() == at::kFloat && k.scalar_type() == at::kFloat &&
+                  v.scalar_type() == at::kFloat && q.is_cuda() && k.is_cuda() &&
+                  v.is_cuda(),
+              "q, k, v must be fp32 GPU tensors");
+  TORCH_CHECK(state.dim() == 4, "state [slots, heads, V, K]");
+  const int heads = state.size(1), V = state.size(2), K = state.size(3);
+  const int tokens = q.size(0), num_seqs = slots.numel();
+  TORCH_CHECK(qk_heads > 0 && heads % qk_heads == 0 &&
+                  q.size(1) == qk_heads * K && k.size(1) == qk_heads * K &&
+                  v.size(1) == heads * V && k.size(0) == tokens &&
+                  v.size(0) == tokens &&
+                  o.numel() == (int64_t)tokens * heads * V &&
+                  positions.numel() >= tokens &&
+                  cu_seqlens.numel() == num_seqs + 1,
+              "linear_scan: shape mismatch");
+  const void *dp = nullptr, *ap = nullptr, *bp = nullptr, *alp = nullptr,
+             *dtp = nullptr;
+  long ab_stride = 0;
+  int ab_f32 = 1;
+  if (decay.has_value()) {
+    CHECK_F32(*decay);
+    TORCH_CHECK(decay->numel() == heads, "decay [heads]");
+    dp = decay->data_ptr();
+  } else {
+    TORCH_CHECK(a_raw.has_value() && b_raw.has_value() && a_log.has_value() &&
+                    dt_bias.has_value(),
+                "the delta form needs a_raw, b_raw, a_log, dt_bias");
+    CHECK_ROWS(*a_raw);
+    CHECK_ROWS(*b_raw);
+    CHECK_F32(*a_log);
+    CHECK_F32(*dt_bias);
+    ab_f32 = act_is_f32(*a_raw, "a_raw");
+    TORCH_CHECK(act_is_f32(*b_raw, "b_raw") == ab_f32 &&
+                    a_raw->size(0) == tokens && b_raw->size(0) == tokens &&
+                    a_raw->size(1) == heads && b_raw->size(1) == heads &&
+                    a_raw->stride(0) == b_raw->stride(0) &&
+                    a_log->numel() == heads && dt_bias->numel() == heads,
+                "linear_scan: a/b shape mismatch");
+    ap = a_raw->data_ptr();
+    bp = b_raw->data_ptr();
+    ab_stride = a_raw->stride(0);
+    alp = a_log->data_ptr();
+    dtp = dt_bias->data_ptr();
+  }
+  check_hip(ks_linear_scan(o.data_ptr(), q.data_ptr(), q.stride(0),
+                           k.data_ptr(), k.stride(0), v.data_ptr(),
+                           v.stride(0), dp, ap, bp, ab_stride, ab_f32, alp, dtp,
+                           state.data_ptr(), positions.data_ptr(),
+                           cu_seqlens.data_ptr(), slots.data_ptr(), num_seqs,
+                           heads, (int)qk_heads, V, K, current_stream()),
+            "linear_scan");
+}
+
 void bias_gelu_tanh(at::Tensor& out, at::Tensor& input, at::Tensor& bias) {
   TORCH_CHECK(input.dim() == 2 && input.is_contiguous() && out.is_contiguous(),
               "input [rows, d] contiguous");
@@ -836,5 +1022,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "per-head matrix product with an optional pair-rotated tail");
   m.def("glu_silu_scale", &glu_silu_scale, "silu(gate) * up * row scale");
   m.def("bias_gelu_tanh", &bias_gelu_tanh, "gelu (tanh form) of x + bias");
+  m.def("relu2_scale", &relu2_scale, "max(x, 0)^2 * row scale");
+  m.def("scale_softcap", &scale_softcap, "cap * tanh(x * scale / cap), fp32");
+  m.def("rope_scale_heads", &rope_scale_heads,
+        "rotary positions on projection heads, times a constant, fp32 out");
+  m.def("unit_norm_heads", &unit_norm_heads,
+        "per-head unit vectors times a constant, in place");
+  m.def("linear_scan", &linear_scan,
+        "decay / gated-delta linear-attention recurrence, per-slot fp32 state");
   def_sampling(m);
 }

@@ -3,7 +3,7 @@
 //  * router_topk: one wave per token. Scores of fp32 logits [T, E] (sigmoid,
 //    or softmax over the experts), the `top` largest chosen one at a time
 //    (ties go to the lower expert), optionally renormalised to sum 1
-//    (divided by their sum + renorm_eps). With a correction vector the
+//    (divided by their sum + renorm_eps) and multiplied by weight_scale. With a correction vector the
 //    choice goes by score + correction[e] while the weights stay the scores.
 //    Outputs expert ids and weights [T, top] and, if asked, the same weights
 //    as a dense [T, E] matrix that is zero for experts not chosen.
@@ -34,7 +34,7 @@ __device__ __forceinline__ void wave_topk(int* __restrict__ idx_out,
                                           const float* z, long t, int E,
                                           int top, int softmax, int renorm,
                                           const float* __restrict__ correction,
-                                          float renorm_eps) {
+                                          float renorm_eps, float weight_scale) {
   const int lane = threadIdx.x & 63;
   float sc[MAX_PER_LANE];  // scores of experts lane + 64 j
   float mx = -INFINITY;
@@ -100,7 +100,8 @@ __device__ __forceinline__ void wave_topk(int* __restrict__ idx_out,
       my_e = be;
     }
   }
-  const float norm = renorm ? 1.0f / (total + renorm_eps) : 1.0f;
+  const float norm =
+      (renorm ? 1.0f / (total + renorm_eps) : 1.0f) * weight_scale;
   if (lane < top) {
     idx_out[t * top + lane] = my_e;
     w_out[t * top + lane] = my_w * norm;
@@ -120,11 +121,11 @@ __global__ void router_topk_kernel(int* __restrict__ idx_out,
                                    const float* __restrict__ logits, int tokens,
                                    int E, int top, int softmax, int renorm,
                                    const float* __restrict__ correction,
-                                   float renorm_eps) {
+                                   float renorm_eps, float weight_scale) {
   const long t = (long)blockIdx.x * NW + (threadIdx.x >> 6);
   if (t >= tokens) return;  // whole waves leave together
   wave_topk(idx_out, w_out, dense_out, logits + t * E, t, E, top, softmax,
-            renorm, correction, renorm_eps);
+            renorm, correction, renorm_eps, weight_scale);
 }
 
 // Router logits and the choice in one kernel: a block per token keeps the
@@ -136,7 +137,7 @@ __global__ void __launch_bounds__(NT) route_tokens_kernel(
     float* __restrict__ dense_out, float* __restrict__ logits_out,
     const T* __restrict__ h, long h_stride, const float* __restrict__ router,
     int W, int E, int top, int softmax, int renorm,
-    const float* __restrict__ correction, float renorm_eps) {
+    const float* __restrict__ correction, float renorm_eps, float weight_scale) {
   extern __shared__ float lds[];
   float* row = lds;      // [W]
   float* z = lds + ((W + 3) & ~3);  // [E]
@@ -188,7 +189,7 @@ __global__ void __launch_bounds__(NT) route_tokens_kernel(
   __syncthreads();
   if (wave == 0)
     wave_topk(idx_out, w_out, dense_out, z, t, E, top, softmax, renorm,
-              correction, renorm_eps);
+              correction, renorm_eps, weight_scale);
 }
 
 __device__ __forceinline__ void ld4_any(const short* p, float* v) {
@@ -281,14 +282,15 @@ extern "C" hipError_t ks_router_topk(void* idx_out, void* w_out,
                                      void* dense_out, const void* logits,
                                      int tokens, int E, int top, int softmax,
                                      int renorm, const void* correction,
-                                     float renorm_eps, hipStream_t stream) {
+                                     float renorm_eps, float weight_scale,
+                                     hipStream_t stream) {
   if (tokens == 0) return hipSuccess;
   if (E < 1 || E > 64 * MAX_PER_LANE || top < 1 || top > E || top > 64)
     return hipErrorInvalidValue;
   hipLaunchKernelGGL(router_topk_kernel, dim3(cdiv(tokens, NW)), dim3(NT), 0,
                      stream, (int*)idx_out, (float*)w_out, (float*)dense_out,
                      (const float*)logits, tokens, E, top, softmax, renorm,
-                     (const float*)correction, renorm_eps);
+                     (const float*)correction, renorm_eps, weight_scale);
   HIP_CHECK_KERNEL();
   return hipSuccess;
 }
@@ -298,7 +300,7 @@ extern "C" hipError_t ks_route_tokens(void* idx_out, void* w_out,
                                       const void* h, long h_stride,
                                       const void* router, int tokens, int W,
                                       int E, int top, int softmax, int renorm,
-                                      const void* correction, float renorm_eps,
+                                      const void* correction, float renorm_eps, float weight_scale,
                                       int is_f32, hipStream_t stream) {
   if (tokens == 0) return hipSuccess;
   if (E < 1 || E > 64 * MAX_PER_LANE || top < 1 || top > E || top > 64 ||
@@ -316,7 +318,7 @@ extern "C" hipError_t ks_route_tokens(void* idx_out, void* w_out,
                        stream, (int*)idx_out, (float*)w_out, (float*)dense_out,
                        (float*)logits_out, (const float*)h, h_stride,
                        (const float*)router, W, E, top, softmax, renorm,
-                       (const float*)correction, renorm_eps);
+                       (const float*)correction, renorm_eps, weight_scale);
   } else {
     if (smem > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(
@@ -328,7 +330,7 @@ extern "C" hipError_t ks_route_tokens(void* idx_out, void* w_out,
                        stream, (int*)idx_out, (float*)w_out, (float*)dense_out,
                        (float*)logits_out, (const short*)h, h_stride,
                        (const float*)router, W, E, top, softmax, renorm,
-                       (const float*)correction, renorm_eps);
+                       (const float*)correction, renorm_eps, weight_scale);
   }
   HIP_CHECK_KERNEL();
   return hipSuccess;

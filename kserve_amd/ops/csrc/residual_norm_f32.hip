@@ -16,7 +16,9 @@
 //    OUTPUT), then either out = residual in the activation dtype (the next
 //    sublayer reads the stream itself) or out = LayerNorm(residual) *
 //    next_weight (the model's final norm). Variances are two-pass.
-//  * gated_group_rms_norm: v = y * silu(z), normalised separately in equal
+//  * gated_group_rms_norm (gate_after set: the norm of y first, the gate on
+//    the normed value; a weight shorter than the row repeats; no weight = 1)
+//    otherwise: v = y * silu(z), normalised separately in equal
 //    contiguous groups of the row, times a weight (gate before the norm).
 //
 // Everything is accumulated in fp32 with exact (non-approximate) sqrt and
@@ -421,35 +423,39 @@ __global__ void gated_group_rms_norm_kernel(TO* __restrict__ out,
                                             const TZ* __restrict__ z,
                                             long z_stride,
                                             const float* __restrict__ weight,
-                                            float eps, int inner,
-                                            int group_size) {
+                                            int weight_n, float eps, int inner,
+                                            int group_size, int gate_after) {
   __shared__ float scratch[NW];
   const long row = blockIdx.x;
   const int g0 = blockIdx.y * group_size;
   float ss = 0.f;
   for (int i = threadIdx.x; i < group_size; i += NT) {
     const float zf = ld_f32(z, row * z_stride + g0 + i);
-    const float v = y[row * inner + g0 + i] * (zf / (1.0f + expf(-zf)));
+    const float yv = y[row * inner + g0 + i];
+    const float v = gate_after ? yv : yv * (zf / (1.0f + expf(-zf)));
     ss += v * v;
   }
   ss = block_sum_sync<NW>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)group_size + eps);
   for (int i = threadIdx.x; i < group_size; i += NT) {
     const float zf = ld_f32(z, row * z_stride + g0 + i);
-    const float v = y[row * inner + g0 + i] * (zf / (1.0f + expf(-zf)));
-    st_f32(out, row * inner + g0 + i, v * inv * weight[g0 + i]);
+    const float gate = zf / (1.0f + expf(-zf));
+    const float yv = y[row * inner + g0 + i];
+    const float w = weight ? weight[(g0 + i) % weight_n] : 1.0f;
+    st_f32(out, row * inner + g0 + i,
+           gate_after ? yv * inv * w * gate : yv * gate * inv * w);
   }
 }
 
 template <typename TZ, typename TO>
 __global__ void gated_group_rms_norm_vec4_kernel(
     TO* __restrict__ out, const float* __restrict__ y, const TZ* __restrict__ z,
-    long z_stride, const float* __restrict__ weight, float eps, int inner,
-    int group_size) {
+    long z_stride, const float* __restrict__ weight, int weight_n, float eps,
+    int inner, int group_size, int gate_after) {
   __shared__ float scratch[NW];
   const long row = blockIdx.x;
   const int g0 = blockIdx.y * group_size;
-  float keep[VEC_STEPS][4];
+  float keep[VEC_STEPS][4], gate[VEC_STEPS][4];
   float ss = 0.f;
 #pragma unroll
   for (int k = 0; k < VEC_STEPS; ++k) {
@@ -460,7 +466,9 @@ __global__ void gated_group_rms_norm_vec4_kernel(
       ld4<TZ>(z + row * z_stride + g0 + i, zv);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float v = yv[j] * (zv[j] / (1.0f + expf(-zv[j])));
+        const float sg = zv[j] / (1.0f + expf(-zv[j]));
+        const float v = gate_after ? yv[j] : yv[j] * sg;
+        gate[k][j] = gate_after ? sg : 1.0f;
         keep[k][j] = v;
         ss += v * v;
       }
@@ -472,10 +480,10 @@ __global__ void gated_group_rms_norm_vec4_kernel(
   for (int k = 0; k < VEC_STEPS; ++k) {
     const int i = (threadIdx.x + NT * k) * 4;
     if (i < group_size) {
-      float w[4], o[4];
-      ld4<float>(weight + g0 + i, w);
+      float w[4] = {1.f, 1.f, 1.f, 1.f}, o[4];
+      if (weight) ld4<float>(weight + (g0 + i) % weight_n, w);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o[j] = keep[k][j] * inv * w[j];
+      for (int j = 0; j < 4; ++j) o[j] = keep[k][j] * inv * w[j] * gate[k][j];
       st4<TO>(out + row * inner + g0 + i, o);
     }
   }
@@ -507,18 +515,31 @@ extern "C" hipError_t ks_embed_scale_sinpos(void* out, const void* table,
 extern "C" hipError_t ks_add_rms_norm_f32res(
     void* residual, const void* d0, long d0_stride, float s0, const void* d1,
     long d1_stride, float s1, const void* weight, float w_offset, float eps,
-    void* out, int rows, int width, int is_f32, hipStream_t stream) {
+    void* out, int rows, int width, int is_f32, int d_is_f32,
+    hipStream_t stream) {
   if (rows == 0) return hipSuccess;
   const int esz = is_f32 ? 4 : 2;
+  const int dsz = d_is_f32 ? 4 : 2;
   auto al = [](const void* p, int bytes) { return ((uintptr_t)p % bytes) == 0; };
   const bool vec = width % 4 == 0 && width <= NT * 4 * VEC_STEPS &&
                    d0_stride % 4 == 0 && d1_stride % 4 == 0 &&
-                   al(residual, 16) && al(weight, 16) && al(d0, 4 * esz) &&
-                   al(d1, 4 * esz) && al(out, 4 * esz);
+                   al(residual, 16) && al(weight, 16) && al(d0, 4 * dsz) &&
+                   al(d1, 4 * dsz) && al(out, 4 * esz);
 #define NORM_ARGS(TT)                                                         \
   (float*)residual, (const TT*)d0, d0_stride, s0, (const TT*)d1, d1_stride,   \
       s1, (const float*)weight, w_offset, eps, (TT*)out, width
-  if (is_f32) {
+#define NORM_ARGS_MIXED                                                       \
+  (float*)residual, (const float*)d0, d0_stride, s0, (const float*)d1,        \
+      d1_stride, s1, (const float*)weight, w_offset, eps, (short*)out, width
+  if (!is_f32 && d_is_f32) {
+    // fp32 deltas (an fp32 sum of sublayer outputs) beside a bf16 output
+    if (vec)
+      hipLaunchKernelGGL((add_rms_norm_f32res_vec4_kernel<float, short>),
+                         dim3(rows), dim3(NT), 0, stream, NORM_ARGS_MIXED);
+    else
+      hipLaunchKernelGGL((add_rms_norm_f32res_kernel<float, short>), dim3(rows),
+                         dim3(NT), 0, stream, NORM_ARGS_MIXED);
+  } else if (is_f32) {
     if (vec)
       hipLaunchKernelGGL((add_rms_norm_f32res_vec4_kernel<float, float>),
                          dim3(rows), dim3(NT), 0, stream, NORM_ARGS(float));
@@ -617,21 +638,27 @@ extern "C" hipError_t ks_post_layer_norm_add(
 
 extern "C" hipError_t ks_gated_group_rms_norm(void* out, const void* y,
                                               const void* z, long z_stride,
-                                              const void* weight, float eps,
-                                              int rows, int inner, int groups,
+                                              const void* weight, int weight_n,
+                                              float eps, int rows, int inner,
+                                              int groups, int gate_after,
                                               int is_f32,
                                               hipStream_t stream) {
   if (rows == 0) return hipSuccess;
   if (groups <= 0 || inner % groups != 0) return hipErrorInvalidValue;
   const int gs = inner / groups;
+  // a weight shorter than the row repeats (one weight vector per group)
+  if (weight && (weight_n <= 0 || inner % weight_n != 0 ||
+                 (weight_n != inner && weight_n % gs != 0 && gs % weight_n != 0)))
+    return hipErrorInvalidValue;
   const int esz = is_f32 ? 4 : 2;
   const bool vec = gs % 4 == 0 && gs <= NT * 4 * VEC_STEPS && z_stride % 4 == 0 &&
+                   (!weight || weight_n % 4 == 0) &&
                    ((uintptr_t)y % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
                    ((uintptr_t)z % (4 * esz)) == 0 &&
                    ((uintptr_t)out % (4 * esz)) == 0;
 #define GNORM_ARGS(TT)                                                        \
   (TT*)out, (const float*)y, (const TT*)z, z_stride, (const float*)weight,    \
-      eps, inner, gs
+      weight_n, eps, inner, gs, gate_after
   if (is_f32) {
     if (vec)
       hipLaunchKernelGGL((gated_group_rms_norm_vec4_kernel<float, float>),

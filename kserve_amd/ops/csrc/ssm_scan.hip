@@ -8,7 +8,7 @@
 // position 0 ignores whatever its slot held (slots are reused, never cleared).
 //
 //  * causal_conv_silu: depthwise causal convolution over `taps` inputs per
-//    channel + bias + silu. Inputs before the portion come from the conv
+//    channel + bias (optional) + silu. Inputs before the portion come from the conv
 //    state (the last taps-1 raw inputs of the sequence), zeros before
 //    position 0.
 //  * conv_state_update: runs after the above, shifts the new raw inputs in.
@@ -64,7 +64,7 @@ __global__ void causal_conv_silu_kernel(
   const long pos = positions[t];
   const long slot = slots[s];
   const int hist = taps - 1;
-  float acc = bias[c];
+  float acc = bias ? bias[c] : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int back = hist - j;  // 0 = the current token
     if (pos - back < 0) continue;
@@ -112,7 +112,8 @@ __global__ void causal_conv_silu_vec4_kernel(
   constexpr int hist = TAPS - 1;
   // taps and bias of this lane's 4 channels, reused for every token
   float wt[4][TAPS], b4[4];
-  load4<float>(bias + c, b4);
+  if (bias) load4<float>(bias + c, b4);
+  else b4[0] = b4[1] = b4[2] = b4[3] = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll

@@ -347,12 +347,20 @@ def add_rms_norm_f32res(
     return (residual * inv * (w_offset + weight)).to(out_dtype)
 
 
-def gated_group_rms_norm(y, z, weight, eps, groups: int, out_dtype):
+def gated_group_rms_norm(
+    y, z, weight, eps, groups: int, out_dtype, gate_after: bool = False
+):
     zf = z.float()
-    v = y * (zf * torch.sigmoid(zf))
+    gate = zf * torch.sigmoid(zf)
+    v = y if gate_after else y * gate
     vg = v.reshape(v.shape[0], groups, -1)
     vg = vg * torch.rsqrt(vg.pow(2).mean(-1, keepdim=True) + eps)
-    return (vg.reshape(v.shape) * weight).to(out_dtype)
+    out = vg.reshape(v.shape)
+    if weight is not None:
+        out = out * weight.repeat(v.shape[1] // weight.numel())
+    if gate_after:
+        out = out * gate
+    return out.to(out_dtype)
 
 
 def causal_conv_silu(x_in, w, bias, conv_state, positions, cu_seqlens, slots):
@@ -371,7 +379,11 @@ def causal_conv_silu(x_in, w, bias, conv_state, positions, cu_seqlens, slots):
             if start - hist + i < 0:
                 prev[i] = 0
         full = torch.cat([prev, x_in[a:b].float()], dim=0)
-        acc = bias.unsqueeze(0).expand(b - a, -1).clone()
+        acc = (
+            bias.unsqueeze(0).expand(b - a, -1).clone()
+            if bias is not None
+            else torch.zeros(b - a, x_in.shape[1])
+        )
         for j in range(taps):
             acc = acc + full[j : j + b - a] * w[:, j].unsqueeze(0)
         out[a:b] = acc * torch.sigmoid(acc)
@@ -518,8 +530,12 @@ def qk_headnorm_rope_cache(
     qf = q.float().reshape(T, heads, D)
     kf = k.float().reshape(T, G, D)
     vf = v.float().reshape(T, G, DV)
-    qn = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * qw
-    kn = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * kw
+    qn = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps)
+    kn = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps)
+    if qw is not None:
+        qn = qn * qw
+    if kw is not None:
+        kn = kn * kw
     if qk_inv_freq is not None:
         qn = rotate_halves(qn, positions, qk_inv_freq)
         kn = rotate_halves(kn, positions, qk_inv_freq)
@@ -561,6 +577,7 @@ def post_norm_add_rms_norm(
 def router_topk(
     logits, top: int, softmax: bool = False, renorm: bool = False,
     dense: bool = False, correction=None, renorm_eps: float = 0.0,
+    weight_scale: float = 1.0,
 ):
     """Scores (sigmoid, or softmax over the experts) of fp32 router logits
     [T, E]; the ``top`` largest per token -> (indices int32 [T, top],
@@ -577,6 +594,8 @@ def router_topk(
         w = torch.gather(s, 1, idx)
     if renorm:
         w = w / (w.sum(-1, keepdim=True) + renorm_eps)
+    if weight_scale != 1.0:
+        w = w * weight_scale
     dw = torch.zeros_like(s).scatter_(1, idx, w) if dense else None
     return idx.to(torch.int32), w, dw
 
@@ -584,14 +603,15 @@ def router_topk(
 def route_tokens(
     h, router, top: int, softmax: bool = False, renorm: bool = False,
     dense: bool = False, want_logits: bool = False, correction=None,
-    renorm_eps: float = 0.0,
+    renorm_eps: float = 0.0, weight_scale: float = 1.0,
 ):
     """Router logits h @ router^T in fp32 (h in the activation dtype, router
     fp32 [E, W]) followed by ``router_topk``; returns (indices, weights,
     dense weights or None, logits or None)."""
     logits = torch.nn.functional.linear(h.float(), router.float())
     idx, w, dw = router_topk(
-        logits, top, softmax, renorm, dense, correction, renorm_eps
+        logits, top, softmax, renorm, dense, correction, renorm_eps,
+        weight_scale,
     )
     return idx, w, dw, (logits if want_logits else None)
 
@@ -730,3 +750,86 @@ def bias_gelu_tanh(x, bias):
     z = x.float() + bias.float()
     y = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
     return y.to(x.dtype)
+
+
+def rope_scale_heads(x, positions, inv_freq, heads_a, scale_a, heads_b, scale_b, dim):
+    """fp32 copy of x [T, width]; rotary positions (pairs i, i + half) on the
+    first heads_a + heads_b heads of ``dim`` columns, the first run times
+    scale_a, the second times scale_b; the remaining columns unchanged."""
+    T = x.shape[0]
+    out = x.float().clone()
+    n = (heads_a + heads_b) * dim
+    if n:
+        xf = out[:, :n].reshape(T, heads_a + heads_b, dim)
+        if inv_freq is not None:
+            xf = rotate_halves(xf, positions, inv_freq)
+        sc = torch.cat(
+            [torch.full((heads_a,), float(scale_a)), torch.full((heads_b,), float(scale_b))]
+        ).view(1, -1, 1)
+        out[:, :n] = (xf * sc).reshape(T, n)
+    return out
+
+
+def unit_norm_heads(x, heads_a, scale_a, heads_b, scale_b, dim, eps):
+    """In place: heads of ``dim`` columns become unit vectors
+    (x / sqrt(sum x^2 + eps)) times scale_a (first heads_a heads) or scale_b
+    (next heads_b)."""
+    T = x.shape[0]
+    for lo, n, sc in ((0, heads_a, scale_a), (heads_a * dim, heads_b, scale_b)):
+        if n:
+            part = x[:, lo : lo + n * dim].reshape(T, n, dim)
+            part = part * torch.rsqrt(part.pow(2).sum(-1, keepdim=True) + eps) * sc
+            x[:, lo : lo + n * dim] = part.reshape(T, n * dim)
+    return x
+
+
+def linear_scan(
+    q, k, v, state, positions, cu_seqlens, slots, qk_heads, decay=None,
+    a_raw=None, b_raw=None, a_log=None, dt_bias=None,
+):
+    """Token-by-token form of the decay / gated-delta recurrences; state
+    [slots, heads, V, K] fp32 is read (unless the portion starts at position
+    0) and written back."""
+    _, heads, V, K = state.shape
+    T = q.shape[0]
+    rep = heads // qk_heads
+    o = torch.empty(T, heads * V, dtype=torch.float32)
+    cu = cu_seqlens.tolist()
+    if decay is None:
+        sp = a_raw.float() + dt_bias
+        sp = torch.where(sp > 30.0, sp, torch.log1p(torch.exp(sp)))
+        g_all = torch.exp(-torch.exp(a_log) * sp)          # [T, heads]
+        b_all = torch.sigmoid(b_raw.float())
+    for s, slot in enumerate(slots.tolist()):
+        a, b = cu[s], cu[s + 1]
+        if b <= a:
+            continue
+        S = state[slot].clone()                              # [heads, V, K]
+        if int(positions[a]) == 0:
+            S.zero_()
+        for t in range(a, b):
+            qt = q[t].float().reshape(qk_heads, K).repeat_interleave(rep, dim=0)
+            kt = k[t].float().reshape(qk_heads, K).repeat_interleave(rep, dim=0)
+            vt = v[t].float().reshape(heads, V)
+            if decay is not None:
+                S = decay[:, None, None] * S + vt[:, :, None] * kt[:, None, :]
+            else:
+                S = g_all[t][:, None, None] * S
+                u = b_all[t][:, None] * (vt - (S * kt[:, None, :]).sum(-1))
+                S = S + u[:, :, None] * kt[:, None, :]
+            o[t] = (S * qt[:, None, :]).sum(-1).reshape(-1)
+        state[slot] = S
+    return o
+
+
+def relu2_scale(x, scales=None):
+    """max(x, 0)^2 (* scales[row]) in x's dtype; arithmetic in fp32."""
+    y = torch.relu(x.float()).pow(2)
+    if scales is not None:
+        y = y * scales.float().view(-1, 1)
+    return y.to(x.dtype)
+
+
+def scale_softcap(x, scale: float, cap: float):
+    z = x.float() * scale
+    return cap * torch.tanh(z / cap) if cap > 0 else z
