@@ -180,6 +180,56 @@ def _voborax_model_configs(size: dict):
     return voborax, desalix
 
 
+# layer shapes for --laperax-compare: the widths, head counts and head sizes
+# of HYBRID_SIZES; value heads of 128 columns over half as many q/k heads in
+# the delta layers, a 1024-token window, 8 experts of which a token uses 2
+LAPERAX_SIZES = {
+    "2k": dict(hybrid="2k", width=2048, heads=16, kv_heads=4, head_dim=128,
+               ff=4096, experts=8, top=2, window=1024, vocab=32000),
+    "4k": dict(hybrid="4k", width=4096, heads=32, kv_heads=8, head_dim=128,
+               ff=7168, experts=8, top=2, window=1024, vocab=32000),
+}
+
+
+def _laperax_model_configs(size: dict):
+    """A four-layer Laperax model (delta, retention, windowed attention,
+    retention; experts beside every mixer) and the Merulorn model that
+    --hybrid-compare measures at the same width."""
+    from kserve_amd.engine.config import (
+        AttentionMixerSpec,
+        DeltaMixerSpec,
+        HybridLayerSpec,
+        HybridModelConfig,
+        RetentionMixerSpec,
+        SquaredReluMoESpec,
+    )
+
+    H, D = size["heads"], size["head_dim"]
+    moe = SquaredReluMoESpec(experts=size["experts"], top=size["top"],
+                             ff=size["ff"], scale=2.5)
+    delta = DeltaMixerSpec(heads=H, kv_heads=H // 2, dim=D, vdim=D, conv=4)
+    ret = RetentionMixerSpec(
+        heads=H, dim=D, vdim=D, rot_dims=D, rot_base=1e6,
+        decay=[1.0 - 2.0 ** (-5.0 - 6.0 * i / max(H - 1, 1)) for i in range(H)],
+    )
+    attn = AttentionMixerSpec(heads=H, kv_heads=size["kv_heads"], dim=D, vdim=D,
+                              scale=D ** -0.5, rot_dims=D // 2, rot_base=1e4,
+                              window=size["window"])
+    layers = [
+        HybridLayerSpec("delta", delta=delta, mlp=moe),
+        HybridLayerSpec("retention", retention=ret, mlp=moe),
+        HybridLayerSpec("attention", attention=attn, mlp=moe),
+        HybridLayerSpec("retention", retention=ret, mlp=moe),
+    ]
+    laperax = HybridModelConfig(
+        vocab_size=size["vocab"], hidden_size=size["width"], layers=layers,
+        model_name="laperax-bench", architecture="Laperax",
+        logit_scale=0.5, logit_softcap=30.0,
+    )
+    merulorn, _ = _hybrid_model_configs(HYBRID_SIZES[size["hybrid"]], layers=4)
+    return laperax, merulorn
+
+
 def _throughput(mcfg, prompt_len, n_prompts, concurrency, steps, warmup, eager):
     """(prefill tok/s, decode tok/s) through the engine's own step()."""
     import torch
@@ -377,6 +427,58 @@ def voborax_compare(args):
     return 0
 
 
+def laperax_compare(args):
+    """Prefill and decode tok/s of the Laperax design next to the Merulorn
+    model of equal width and depth (the closest design the engine serves:
+    recurrent state per slot beside KV pages, a scan kernel, a short
+    convolution), both through LLMEngine.step() on one GPU, bf16, random
+    weights. One JSON line per (size, model), each measured in a process of
+    its own."""
+    import subprocess
+    import sys
+
+    if args.compare_only is None or "," in args.laperax_compare:
+        rc = 0
+        for name in args.laperax_compare.split(","):
+            for label in ("laperax", "merulorn"):
+                if args.compare_only and args.compare_only != label:
+                    continue
+                cmd = [sys.executable, "-u", os.path.abspath(__file__),
+                       "--laperax-compare", name, "--compare-only", label,
+                       "--steps", str(args.steps), "--warmup", str(args.warmup),
+                       "--concurrency", str(args.concurrency),
+                       "--prompt-len", str(args.prompt_len)]
+                if args.eager:
+                    cmd.append("--eager")
+                rc = subprocess.call(cmd)
+                if rc != 0:
+                    return rc
+        return rc
+
+    import torch
+
+    assert torch.cuda.is_available(), "--laperax-compare needs a GPU"
+    name, label = args.laperax_compare, args.compare_only
+    size = LAPERAX_SIZES[name]
+    laperax, merulorn = _laperax_model_configs(size)
+    mcfg = laperax if label == "laperax" else merulorn
+    prefill, decode = _throughput(
+        mcfg, prompt_len=args.prompt_len if args.prompt_len != 512 else 2048,
+        n_prompts=8, concurrency=min(args.concurrency, 256),
+        steps=args.steps, warmup=args.warmup, eager=args.eager,
+    )
+    print(json.dumps({
+        "bench": "laperax-compare", "size": name, "model": mcfg.model_name,
+        "layers": 4, "width": size["width"],
+        "prefill_tok_s": round(prefill, 1),
+        "decode_tok_s": round(decode, 1),
+        "prefill_batch": "8 x prompt", "decode_concurrency":
+            min(args.concurrency, 256),
+        "dtype": "bfloat16", "data": "synthetic, random-init weights",
+    }), flush=True)
+    return 0
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -429,10 +531,18 @@ def main():
                              "beside the Desalix model of equal width, heads, "
                              "depth and experts (sizes: "
                              + ", ".join(VOBORAX_SIZES) + ")")
+    parser.add_argument("--laperax-compare", type=str, default=None,
+                        metavar="SIZE[,SIZE...]",
+                        help="instead of the flagship workload: prefill and "
+                             "decode throughput of a Laperax-design model "
+                             "beside the Merulorn model of equal width and "
+                             "depth (sizes: " + ", ".join(LAPERAX_SIZES) + ")")
     parser.add_argument("--compare-only", type=str, default=None,
-                        choices=["desalix", "llama", "voborax"],
-                        help="with --desalix-compare / --voborax-compare: run "
-                             "one side only (e.g. under a profiler)")
+                        choices=["desalix", "llama", "voborax", "laperax",
+                                 "merulorn"],
+                        help="with --desalix-compare / --voborax-compare / "
+                             "--laperax-compare: run one side only (e.g. "
+                             "under a profiler)")
     parser.add_argument("--profile-cpu", action="store_true",
                         help="cProfile the timed loop and print hot functions")
     args = parser.parse_args()
@@ -442,6 +552,8 @@ def main():
         return desalix_compare(args)
     if args.voborax_compare:
         return voborax_compare(args)
+    if args.laperax_compare:
+        return laperax_compare(args)
 
     import torch
 

@@ -366,6 +366,9 @@ extern "C" hipError_t ks_linear_scan(
   const int R = cdiv(K, 16);
   int pc = V > 32 ? 4 : (V > 16 ? 2 : 1);
   if (R > 8 && pc > 2) pc = 2;
+  // a block walks its tokens one after the other, so a launch with few
+  // (sequence, head) pairs takes narrower tiles to put more blocks on the chip
+  while (pc > 1 && (long)cdiv(V, 16 * pc) * heads * num_seqs < 1024) pc >>= 1;
   const int xs = 16 * pc;
   const size_t smem = sizeof(float) * ((size_t)SCAN_TC * (2 * K + 2 * xs + 3));
   dim3 grid(cdiv(V, xs), heads, num_seqs);

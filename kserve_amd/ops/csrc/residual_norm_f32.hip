@@ -489,6 +489,46 @@ __global__ void gated_group_rms_norm_vec4_kernel(
   }
 }
 
+// Groups of at most 256 elements (heads of a recurrent read-out): a block
+// takes a whole row and each of its waves a group at a time, 4 elements per
+// lane, so a row costs one block instead of one block per group.
+template <typename TZ, typename TO>
+__global__ void __launch_bounds__(NT) gated_group_rms_norm_wave_kernel(
+    TO* __restrict__ out, const float* __restrict__ y, const TZ* __restrict__ z,
+    long z_stride, const float* __restrict__ weight, int weight_n, float eps,
+    int inner, int group_size, int groups, int gate_after) {
+  const long row = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int i = lane * 4;
+  const bool on = i < group_size;
+  for (int g = threadIdx.x >> 6; g < groups; g += NW) {
+    const int g0 = g * group_size;
+    float v[4] = {0.f, 0.f, 0.f, 0.f}, gate[4] = {1.f, 1.f, 1.f, 1.f};
+    float ss = 0.f;
+    if (on) {
+      float zv[4];
+      ld4<float>(y + row * inner + g0 + i, v);
+      ld4<TZ>(z + row * z_stride + g0 + i, zv);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float sg = zv[j] / (1.0f + expf(-zv[j]));
+        if (gate_after) gate[j] = sg;
+        else v[j] *= sg;
+        ss += v[j] * v[j];
+      }
+    }
+    ss = wave_reduce_sum(ss);
+    if (on) {
+      const float inv = 1.0f / sqrtf(ss / (float)group_size + eps);
+      float w[4] = {1.f, 1.f, 1.f, 1.f}, o[4];
+      if (weight) ld4<float>(weight + (g0 + i) % weight_n, w);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = v[j] * inv * w[j] * gate[j];
+      st4<TO>(out + row * inner + g0 + i, o);
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" hipError_t ks_embed_scale_sinpos(void* out, const void* table,
@@ -658,25 +698,37 @@ extern "C" hipError_t ks_gated_group_rms_norm(void* out, const void* y,
                    ((uintptr_t)out % (4 * esz)) == 0;
 #define GNORM_ARGS(TT)                                                        \
   (TT*)out, (const float*)y, (const TT*)z, z_stride, (const float*)weight,    \
-      weight_n, eps, inner, gs, gate_after
+      weight_n, eps, inner, gs
+  if (vec && gs <= 4 * WAVE_SIZE && groups > 1) {
+    if (is_f32)
+      hipLaunchKernelGGL((gated_group_rms_norm_wave_kernel<float, float>),
+                         dim3(rows), dim3(NT), 0, stream, GNORM_ARGS(float),
+                         groups, gate_after);
+    else
+      hipLaunchKernelGGL((gated_group_rms_norm_wave_kernel<short, short>),
+                         dim3(rows), dim3(NT), 0, stream, GNORM_ARGS(short),
+                         groups, gate_after);
+    HIP_CHECK_KERNEL();
+    return hipSuccess;
+  }
   if (is_f32) {
     if (vec)
       hipLaunchKernelGGL((gated_group_rms_norm_vec4_kernel<float, float>),
                          dim3(rows, groups), dim3(NT), 0, stream,
-                         GNORM_ARGS(float));
+                         GNORM_ARGS(float), gate_after);
     else
       hipLaunchKernelGGL((gated_group_rms_norm_kernel<float, float>),
                          dim3(rows, groups), dim3(NT), 0, stream,
-                         GNORM_ARGS(float));
+                         GNORM_ARGS(float), gate_after);
   } else {
     if (vec)
       hipLaunchKernelGGL((gated_group_rms_norm_vec4_kernel<short, short>),
                          dim3(rows, groups), dim3(NT), 0, stream,
-                         GNORM_ARGS(short));
+                         GNORM_ARGS(short), gate_after);
     else
       hipLaunchKernelGGL((gated_group_rms_norm_kernel<short, short>),
                          dim3(rows, groups), dim3(NT), 0, stream,
-                         GNORM_ARGS(short));
+                         GNORM_ARGS(short), gate_after);
   }
   HIP_CHECK_KERNEL();
   return hipSuccess;
