@@ -525,6 +525,26 @@ class TestPlumbing:
         assert set(layout[1][1]) == {"ssm"}
         assert layout[1][1]["ssm"][0] == (2, 12, 8)
 
+    def test_server_cli_picks_the_engine(self, tmp_path):
+        from kserve_amd.runtimes.huggingfaceserver import detect_backend
+
+        (tmp_path / "config.json").write_text(json.dumps(three_kinds_config()))
+        assert detect_backend(str(tmp_path)) == "engine"
+
+    def test_unknown_parts_are_refused(self):
+        cfg = three_kinds_config()
+        cfg["layers"][0]["type"] = "something-else"
+        with pytest.raises(ValueError):
+            HybridModelConfig.from_dict(cfg)
+        cfg = three_kinds_config()
+        cfg["layers"][0]["mlp"]["kind"] = "dense"
+        with pytest.raises(ValueError):
+            HybridModelConfig.from_dict(cfg)
+        cfg = three_kinds_config()
+        cfg["layers"][1]["mixer"]["decay"] = [0.5]
+        with pytest.raises(ValueError):
+            HybridModelConfig.from_dict(cfg)
+
     def test_engine_from_a_model_directory(self, tmp_path):
         from safetensors.torch import save_file
 
