@@ -62,8 +62,11 @@ class SchedulerMachine(RuleBasedStateMachine):
             for req, n in zip(batch.requests, batch.num_scheduled_tokens):
                 assert n > 0
                 req.num_computed_tokens += n
-                if req.num_computed_tokens >= req.num_prompt_tokens:
-                    # prompt done: first output token materializes
+                # the engine's rule: a (re-)prefill is done when every token
+                # the request holds is computed; after a recompute preemption
+                # that includes the tokens generated before it
+                if req.num_computed_tokens >= req.num_tokens:
+                    # prompt done: the next output token materializes
                     req.output_token_ids.append(7)
                 else:
                     # chunked: back to waiting for the next chunk
