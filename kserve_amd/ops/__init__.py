@@ -317,6 +317,8 @@ def topk_topp_sample_into(
     """Destination-passing form of the fused sampler for hipGraph capture
     (static out buffer, per-row device seeds; see model_runner
     _ensure_sampled_graph). GPU-only."""
+    if logits.dtype != torch.bfloat16:
+        logits = logits.to(torch.bfloat16)  # the fused samplers' format
     _native_sampling("random_sample").topk_topp_sample(
         out, logits, temperatures, top_p,
         top_k if top_k.dtype == torch.int32 else top_k.to(torch.int32),

@@ -497,6 +497,25 @@ class TestGeneration:
             assert eng.scheduler.state_slots.num_free == kw.get("max_seqs", 4)
 
 
+    def test_sampled_generation(self, backend):
+        """Temperature sampling through the engine's samplers (on the GPU the
+        fused sampler inside captured multi-step windows): the model hands
+        over fp32 logits in both activation dtypes."""
+        cfg = three_kinds_config()
+        sd = weights_for(cfg, backend, seed=31)
+        prompts = [random_prompt(n, cfg["vocab"], 80 + n) for n in (9, 4, 15)]
+        eng = make_engine(cfg, sd, backend, multi_step=4)
+        outs = eng.generate(
+            prompts,
+            SamplingParams(max_tokens=10, temperature=0.8, top_k=20, top_p=0.9,
+                           ignore_eos=True, seed=5),
+        )
+        assert len(outs) == 3
+        for o in outs.values():
+            assert len(o.output_token_ids) == 10
+            assert all(0 <= t < cfg["vocab"] for t in o.output_token_ids)
+
+
 class TestPlumbing:
     def test_registry_config_layout_and_loading(self, tmp_path):
         from safetensors.torch import save_file
